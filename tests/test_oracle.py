@@ -1,0 +1,251 @@
+"""Pins for the CPU oracle.  None of these re-type the oracle's own formula: each
+compares it with an independent statement (python/numpy float64 loops, a torch
+library routine, autograd, a closed form or an invariant)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import gca_oracle as orc
+
+
+def _rand(*shape, seed=0, scale=1.0, dtype=torch.float64):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g, dtype=torch.float64) * scale).to(dtype)
+
+
+# ----------------------------------------------------------------------------- retrieval
+
+def test_scores_vs_loops():
+    N, C, E, D = 2, 3, 5, 7
+    a, b = _rand(N, C, D, seed=1), _rand(N, E, D, seed=2)
+    got = orc.landmark_scores(a, b, hidden_size=D)
+    an, bn = a.numpy(), b.numpy()
+    for n in range(N):
+        for c in range(C):
+            for e in range(E):
+                ref = sum(an[n, c, i] * bn[n, e, i] for i in range(D)) / math.sqrt(D)
+                assert abs(got[n, c, e].item() - ref) < 1e-12
+    # divisor is the argument, not the head dim
+    assert torch.allclose(orc.landmark_scores(a, b, hidden_size=4 * D) * 2, got)
+
+
+@pytest.mark.parametrize("dec,enc", [(4, 4), (1, 6), (3, 5), (5, 5)])
+def test_causal_mask_vs_loops(dec, enc):
+    vis = orc.causal_visible(dec, enc)
+    assert vis.shape == (dec, enc)
+    for r in range(dec):
+        dec_id = enc - dec + r          # last `dec` ids of arange(enc)
+        for e in range(enc):
+            assert bool(vis[r, e]) == (dec_id > e)
+    if dec == enc:
+        assert not vis[0].any()          # first row sees nothing (strict past)
+    win = orc.causal_visible(dec, enc, max_chunk_win=2)
+    for r in range(dec):
+        dec_id = enc - dec + r
+        for e in range(enc):
+            assert bool(win[r, e]) == (dec_id > e and dec_id <= e + 2)
+
+
+def test_topk_equals_torch_topk_on_distinct_values():
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(6, 9, 300, generator=g)
+    v, i = orc.topk_canonical(x, 8)
+    tv, ti = torch.topk(x, 8, dim=-1)
+    assert torch.equal(v, tv) and torch.equal(i, ti)
+
+
+def test_topk_tie_rule_vs_python_sort():
+    g = torch.Generator().manual_seed(4)
+    x = torch.randint(0, 4, (5, 40), generator=g).float()      # many exact ties
+    x[1, 7:] = float('-inf')
+    x[2, :] = float('-inf')
+    v, i = orc.topk_canonical(x, 6)
+    for r in range(x.shape[0]):
+        order = sorted(range(x.shape[1]), key=lambda e: (-x[r, e].item(), e))[:6]
+        assert i[r].tolist() == order
+        assert v[r].tolist() == [x[r, e].item() for e in order]
+
+
+def test_retrieval_invariants():
+    N, C, D, K = 2, 12, 16, 4
+    lq, lk = _rand(N, C, D, seed=5, dtype=torch.float32), _rand(N, C, D, seed=6, dtype=torch.float32)
+    scores, idx, w = orc.retrieve(lq, lk, K, hidden_size=D)
+    assert idx.shape == (N, C, K) and w.shape == (N, C, K)
+    assert (w >= 0).all()
+    rs = w.sum(-1)
+    assert torch.allclose(rs[:, 0], torch.zeros(N))              # row 0 sees nothing -> all weights 0
+    assert torch.allclose(rs[:, 1:], torch.ones(N, C - 1), atol=1e-6)
+    sel = scores.gather(2, idx)
+    assert (sel[..., :-1] >= sel[..., 1:]).all()                 # slot order: descending
+    assert (w[sel == float('-inf')] == 0).all()                  # masked slots weigh 0
+    for c in range(1, C):                                        # selected finite slots are strictly past
+        fin = sel[:, c] > float('-inf')
+        assert (idx[:, c][fin] < c).all()
+        assert fin.sum(-1).eq(min(c, K)).all()
+    # k' = min(E, chunk_topk)
+    _, idx2, _ = orc.retrieve(lq[:, :3], lk[:, :3], K, hidden_size=D)
+    assert idx2.shape[-1] == 3
+    # Gumbel noise changes the selection only, weights come from noise-free scores
+    noise = _rand(N, C, C, seed=7, dtype=torch.float32) * 5
+    s3, idx3, w3 = orc.retrieve(lq, lk, K, hidden_size=D, noise=noise)
+    assert torch.equal(s3, scores)
+    assert torch.allclose(w3, torch.nan_to_num(F.softmax(scores.gather(2, idx3), -1), nan=0.0))
+    assert not torch.equal(idx3, idx)
+
+
+def test_gather_vs_loops():
+    N, C, S, H, d, K = 2, 5, 3, 2, 4, 3
+    ck, cv = _rand(N, C, S, H * d, seed=8), _rand(N, C, S, H * d, seed=9)
+    g = torch.Generator().manual_seed(10)
+    idx = torch.randint(0, C, (N, C, K), generator=g)
+    w = torch.rand(N, C, K, generator=g, dtype=torch.float64)
+    k, v, ww = orc.gather_chunks(ck, cv, idx, w, H)
+    assert k.shape == (N * (C - 1), H, K, S, d) and ww.shape == (N * (C - 1), K)
+    for n in range(N):
+        for c in range(C - 1):           # retrieval row c (last row dropped)
+            z = n * (C - 1) + c
+            for j in range(K):
+                assert ww[z, j] == w[n, c, j]
+                for h in range(H):
+                    assert torch.equal(k[z, h, j], ck[n, idx[n, c, j], :, h * d:(h + 1) * d])
+                    assert torch.equal(v[z, h, j], cv[n, idx[n, c, j], :, h * d:(h + 1) * d])
+
+
+# ----------------------------------------------------------------------------- forward
+
+def _inputs(Z=2, Hq=4, Hkv=2, K=3, Q=5, S=6, d=4, seed=0, dtype=torch.float64):
+    q = _rand(Z, Hq, Q, d, seed=seed, scale=0.7, dtype=dtype)
+    k = _rand(Z, Hkv, K, S, d, seed=seed + 1, scale=0.7, dtype=dtype)
+    v = _rand(Z, Hkv, K, S, d, seed=seed + 2, scale=0.7, dtype=dtype)
+    w = torch.softmax(_rand(Z, K, seed=seed + 3, dtype=dtype), -1)
+    return q, k, v, w
+
+
+@pytest.mark.parametrize("sm_n", [0.0, 1.0, 2.5])
+def test_forward_vs_numpy_loops(sm_n):
+    q, k, v, w = _inputs()
+    Z, Hq, Q, d = q.shape
+    Hkv, K, S = k.shape[1], k.shape[2], k.shape[3]
+    G = Hq // Hkv
+    scale = 0.37
+    got = orc.gca_forward(q, k, v, w, scale, sm_n).numpy()
+    qn, kn, vn, wn = q.numpy(), k.numpy(), v.numpy(), w.numpy()
+    for z in range(Z):
+        for h in range(Hq):
+            hk = h // G
+            for m in range(Q):
+                out = np.zeros(d)
+                for j in range(K):
+                    e = np.array([math.exp(scale * float(qn[z, h, m] @ kn[z, hk, j, n])) for n in range(S)])
+                    p = e / (sm_n + e.sum())
+                    out += wn[z, j] * (p @ vn[z, hk, j])
+                assert np.allclose(got[z, h, m], out, rtol=1e-10, atol=1e-12)
+
+
+def test_forward_vs_sdpa_per_chunk():
+    q, k, v, w = _inputs(Z=2, Hq=4, Hkv=4, K=3, Q=8, S=8, d=16, dtype=torch.float32)
+    scale = 1 / math.sqrt(16)
+    got = orc.gca_forward(q, k, v, w, scale, 0.0)
+    ref = torch.zeros_like(q)
+    for j in range(k.shape[2]):
+        ref += w[:, j].view(-1, 1, 1, 1) * F.scaled_dot_product_attention(q, k[:, :, j], v[:, :, j], scale=scale)
+    assert torch.allclose(got, ref, atol=1e-5)
+
+
+def test_softmax_one_equals_zero_row_and_closed_form():
+    q, k, v, w = _inputs()
+    scale = 0.5
+    a = orc.gca_forward(q, k, v, w, scale, 1.0)
+    # closed form: one extra zero key and zero value row (what the model does by zeroing the landmark row)
+    zk = torch.zeros_like(k[:, :, :, :1])
+    b = orc.gca_forward(q, torch.cat([k, zk], 3), torch.cat([v, zk], 3), w, scale, 0.0)
+    assert torch.allclose(a, b, rtol=1e-12, atol=1e-14)
+    s = _rand(3, 7, seed=11)
+    assert torch.allclose(orc.softmax_n(s, 1.0), torch.softmax(torch.cat([s, torch.zeros(3, 1, dtype=s.dtype)], -1), -1)[:, :-1])
+    # far-negative scores must not overflow
+    assert torch.isfinite(orc.softmax_n(s - 1000.0, 1.0)).all()
+
+
+def test_forward_special_cases():
+    q, k, v, w = _inputs(K=1, Hq=2, Hkv=2)
+    one = torch.ones_like(w)
+    ref = F.scaled_dot_product_attention(q, k[:, :, 0], v[:, :, 0], scale=0.3)
+    assert torch.allclose(orc.gca_forward(q, k, v, one, 0.3, 0.0), ref)          # K=1, w=1: plain attention
+    q, k, v, w = _inputs(K=4)
+    eq = torch.full_like(w, 0.25)
+    _, o_k, _, _ = orc.gca_forward(q, k, v, eq, 0.3, 0.0, return_parts=True)
+    assert torch.allclose(orc.gca_forward(q, k, v, eq, 0.3, 0.0), o_k.mean(2))   # equal weights: mean
+    vc = torch.full_like(v, 1.5)
+    out = orc.gca_forward(q, k, vc, w, 0.3, 0.0)
+    assert torch.allclose(out, (1.5 * w.sum(-1)).view(-1, 1, 1, 1).expand_as(out))  # constant V
+
+
+def test_lse2_closed_form():
+    q, k, v, w = _inputs()
+    for sm_n in (0.0, 1.0):
+        lse2 = orc.gca_lse2(q, k, 0.4, sm_n)
+        _, _, p, s = orc.gca_forward(q, k, v, w, 0.4, sm_n, return_parts=True)
+        assert torch.allclose(torch.exp2(s * orc.LOG2E - lse2.unsqueeze(-1)), p, rtol=1e-10)
+
+
+# ----------------------------------------------------------------------------- backward
+
+@pytest.mark.parametrize("sm_n", [0.0, 1.0])
+@pytest.mark.parametrize("G", [1, 2])
+def test_backward_vs_autograd(sm_n, G):
+    q, k, v, w = _inputs(Hq=4, Hkv=4 // G)
+    do = _rand(*q.shape, seed=20)
+    dq, dk, dv, dw = orc.gca_backward(q, k, v, w, do, 0.45, sm_n)
+    _, aq, ak, av, aw = orc.gca_forward_backward_autograd(q, k, v, w, do, 0.45, sm_n)
+    for a, b in ((dq, aq), (dk, ak), (dv, av), (dw, aw)):
+        assert torch.allclose(a, b, rtol=1e-9, atol=1e-12)
+
+
+@pytest.mark.parametrize("sm_n", [0.0, 1.0])
+def test_gradcheck_fp64(sm_n):
+    q, k, v, w = _inputs(Z=1, Hq=2, Hkv=1, K=2, Q=3, S=4, d=4)
+    ins = [t.clone().requires_grad_(True) for t in (q, k, v, w)]
+    assert torch.autograd.gradcheck(lambda a, b, c, d_: orc.gca_forward(a, b, c, d_, 0.6, sm_n), ins, eps=1e-6, atol=1e-6)
+
+
+def test_backward_invariants():
+    q, k, v, w = _inputs()
+    do = _rand(*q.shape, seed=21)
+    o, o_k, p, _ = orc.gca_forward(q, k, v, w, 0.45, 1.0, return_parts=True)
+    delta = torch.einsum('zhkmd,zhmd->zhkm', o_k, do)
+    assert torch.allclose(torch.einsum('zhkm,zk->zhm', delta, w), (o * do).sum(-1))   # sum_j w_j D_j = rowsum(O*dO)
+    dq, dk, dv, dw = orc.gca_backward(q, k, v, w, do, 0.45, 1.0)
+    assert torch.allclose(dw, delta.sum((1, 3)))
+    # a slot with weight 0 gets no dk/dv but still a dw
+    w0 = w.clone(); w0[:, 1] = 0
+    _, dk0, dv0, dw0 = orc.gca_backward(q, k, v, w0, do, 0.45, 1.0)
+    assert dk0[:, :, 1].abs().max() == 0 and dv0[:, :, 1].abs().max() == 0 and dw0[:, 1].abs().min() > 0
+
+
+# ----------------------------------------------------------------------------- caller contract
+
+def test_layer_row_shift_and_zero_first_chunk():
+    N, C, H, S, d, K = 2, 6, 2, 4, 8, 3
+    q_all = _rand(N, C, H, S, d, seed=30, dtype=torch.float32)
+    ck, cv = _rand(N, C, S, H * d, seed=31, dtype=torch.float32), _rand(N, C, S, H * d, seed=32, dtype=torch.float32)
+    lq, lk = _rand(N, C, H * d, seed=33, dtype=torch.float32), _rand(N, C, H * d, seed=34, dtype=torch.float32)
+    out, idx, w = orc.gca_layer(q_all, ck, cv, lq, lk, K, H, sm_n=1.0)
+    assert out[:, 0].abs().max() == 0
+    # query chunk c+1 attends the chunks picked by retrieval row c, all strictly before c+1
+    for n in range(N):
+        for c in range(1, C - 1):
+            ref = torch.zeros(H, S, d)
+            for j in range(K):
+                e = int(idx[n, c, j])
+                if w[n, c, j] == 0:
+                    continue
+                assert e < c
+                for h in range(H):
+                    s = (q_all[n, c + 1, h] @ ck[n, e, :, h * d:(h + 1) * d].T) / math.sqrt(d)
+                    ex = torch.exp(s)
+                    p = ex / (1.0 + ex.sum(-1, keepdim=True))
+                    ref[h] += w[n, c, j] * (p @ cv[n, e, :, h * d:(h + 1) * d])
+            assert torch.allclose(out[n, c + 1], ref, atol=1e-5)
