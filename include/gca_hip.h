@@ -1,0 +1,148 @@
+/*
+ * gca_hip.h -- C ABI of libgca_hip.so: Grouped Cross-Attention (GCA) and landmark
+ * retrieval for AMD MI355X (gfx950), hand-written HIP kernels.
+ *
+ * Every entry point takes raw DEVICE pointers to contiguous row-major buffers, plain
+ * integers for sizes and an opaque stream handle (a hipStream_t passed as void*; NULL
+ * is the default stream).  All launches are asynchronous on that stream; nothing here
+ * synchronises the device, allocates or frees device memory, or keeps a pointer after
+ * returning.  Functions are re-entrant and may be called from any host thread (the
+ * autograd engine calls the backward from a worker thread).  Each returns GCA_OK or a
+ * GCA_ERR_* code and never aborts; gca_strerror() names a code.
+ *
+ * "Reference" below is ant-research/long-context-modeling; each entry point cites the
+ * reference interface it replaces (paths relative to that checkout).
+ *
+ * Tensor layouts (element type T = desc.dtype; all contiguous):
+ *   q, o, do, dq      (Z, Hq, Q_CTX, D)
+ *   k, v, dk, dv      (Z, Hkv, K, K_CTX, D)          gathered ("retrieved chunks") form
+ *   weights           (Z, K)      type desc.w_dtype  shared by all heads
+ *   lse               (Z, Hq, K, Q_CTX)  float       log2 of the softmax denominator of the
+ *                                                    log2-scaled scores, per retrieved chunk
+ *   dw                (Z, K)      float
+ *   k_cache, v_cache  (N, C, K_CTX, Hkv*D)           the chunk cache the model keeps
+ *   indices           (Z, K)      int64              chunk ids inside the row's own sequence;
+ *                                                    row z belongs to sequence z / (Z / N)
+ * Query head h reads kv head h / (Hq / Hkv).
+ */
+#ifndef GCA_HIP_H
+#define GCA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum gca_dtype { GCA_F32 = 0, GCA_BF16 = 1 };
+
+enum gca_status {
+    GCA_OK = 0,
+    GCA_ERR_NULL = 1,        /* a required pointer is NULL */
+    GCA_ERR_SHAPE = 2,       /* a size is zero/negative, Hq % Hkv != 0, D not in {16,32,64,128,256}, ... */
+    GCA_ERR_DTYPE = 3,       /* unknown element type */
+    GCA_ERR_LAUNCH = 4,      /* the HIP runtime refused a launch (wrong GPU architecture, ...) */
+    GCA_ERR_WORKSPACE = 5,   /* workspace pointer NULL or too small */
+    GCA_ERR_UNSUPPORTED = 6  /* valid request this build has no kernel for */
+};
+
+/* Which kernel family a call may use.  AUTO picks the MFMA kernels when the shape
+ * qualifies (bf16, K_CTX == 64, D in {64, 128}, Q_CTX % 64 == 0) and the generic
+ * ones otherwise; the other two force a family (MFMA returns GCA_ERR_UNSUPPORTED
+ * when the shape does not qualify). */
+enum gca_path { GCA_PATH_AUTO = 0, GCA_PATH_GENERIC = 1, GCA_PATH_MFMA = 2 };
+
+typedef struct gca_desc {
+    int32_t dtype;      /* gca_dtype of q, k, v, o and their gradients */
+    int32_t w_dtype;    /* gca_dtype of weights */
+    int64_t Z;          /* query chunks: batch x (chunks - 1) in training */
+    int32_t Hq;         /* query heads */
+    int32_t Hkv;        /* key/value heads, divides Hq */
+    int32_t K;          /* retrieved chunks per query chunk (top-k) */
+    int32_t Q_CTX;      /* query rows per chunk (64 in the model; 1 or 2 in decode steps) */
+    int32_t K_CTX;      /* key rows per retrieved chunk (64 in the model) */
+    int32_t D;          /* head dim: 16, 32, 64, 128 or 256 */
+    float sm_scale;     /* multiplies q.k before the softmax */
+    float sm_n;         /* softmax denominator offset: P = exp(s) / (sm_n + sum exp(s)); 0 = plain */
+    int32_t path;       /* gca_path */
+    int32_t reserved;
+    int64_t N;          /* indexed entry points: sequences in the cache (Z % N == 0) */
+    int64_t C;          /* indexed entry points: chunks per sequence in the cache */
+} gca_desc;
+
+typedef struct lmk_desc {
+    int32_t dtype;          /* gca_dtype of lmk_q, lmk_k, scores, noise */
+    int32_t topk;           /* requested k; the kernels emit kk = min(E, topk) slots per row */
+    int64_t N;              /* sequences */
+    int64_t C;              /* query landmarks (rows) per sequence */
+    int64_t E;              /* candidate chunks per sequence */
+    int32_t Dm;             /* landmark width */
+    int32_t causal;         /* 1: row c sees chunk e iff (E - C + c) > e, others are -inf */
+    float hidden_size;      /* scores are divided by sqrt(hidden_size) */
+    int32_t reserved;
+} lmk_desc;
+
+/* Library version (major*10000 + minor*100 + patch) and status text. */
+int gca_version(void);
+const char* gca_strerror(int status);
+
+/* Forward on gathered K/V.  lse may be NULL (inference: nothing is saved).
+ * Replaces _attention.forward (ltriton/gca.py:684-738, kernel _attn_fwd :94-211) and,
+ * with lse == NULL, gca_kv_cache (ltriton/gca.py:846-888, kernel _attn_inf :214-314). */
+int gca_fwd(const gca_desc* desc, const void* q, const void* k, const void* v, const void* weights,
+            void* o, float* lse, void* stream);
+
+/* Bytes of scratch gca_bwd needs (the per-chunk row sums D_j, (Z, Hq, K, Q_CTX) floats). */
+size_t gca_bwd_workspace_bytes(const gca_desc* desc);
+
+/* Backward on gathered K/V: dq, dk, dv in T, dw in float.
+ * Replaces _attention.backward (ltriton/gca.py:741-841; kernels :484-572 and :576-675,
+ * the host-side dw reduction :839-840). */
+int gca_bwd(const gca_desc* desc, const void* q, const void* k, const void* v, const void* weights,
+            const void* dout, const float* lse, void* dq, void* dk, void* dv, float* dw,
+            void* workspace, size_t workspace_bytes, void* stream);
+
+/* Forward reading the retrieved chunks straight from the chunk cache by index, so the
+ * K-times-larger gathered copies are never written.  Replaces
+ * ChunkKVManager.retrieve_chunks (model/DRT.py:193-200) + preprocess_chunk_kv_cache
+ * (model/DRT.py:320-332) + _attention.forward. */
+int gca_fwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, const void* v_cache,
+                    const int64_t* indices, const void* weights, void* o, float* lse, void* stream);
+
+/* Backward of gca_fwd_indexed.  dk_cache / dv_cache are FLOAT buffers of the cache's
+ * shape (N, C, K_CTX, Hkv*D) that the caller has zeroed; gradients of chunks retrieved
+ * by several query chunks are summed into them (the index_put_(accumulate=True) that
+ * autograd runs for model/DRT.py:198-199). */
+int gca_bwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, const void* v_cache,
+                    const int64_t* indices, const void* weights, const void* dout, const float* lse,
+                    void* dq, float* dk_cache, float* dv_cache, float* dw,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* scores[n, c, e] = <lmk_q[n, c, :], lmk_k[n, e, :]> / sqrt(hidden_size), -inf where masked.
+ * lmk_q (N, C, Dm), lmk_k (N, E, Dm), scores (N, C, E), all of desc.dtype.
+ * Replaces model/DRT.py:612-613 (decode copy :838-840). */
+int lmk_score(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, void* scores, void* stream);
+
+/* Bytes of scratch lmk_topk needs for rows of E candidates. */
+size_t lmk_topk_workspace_bytes(const lmk_desc* desc);
+
+/* Top-k selection and retrieval weights over rows of scores.
+ * indices (N, C, kk) int64 in selection order: higher (score + noise) first, ties by lower
+ * index first; weights (N, C, kk) float = softmax over the noise-free masked scores of the
+ * selected slots, NaN -> 0 (a slot holding -inf weighs exactly 0).  noise may be NULL.
+ * When desc.causal is set the mask is applied here as well, so unmasked scores are fine.
+ * Replaces model/DRT.py:613-627 (decode copy :840-844). */
+int lmk_topk(const lmk_desc* desc, const void* scores, const void* noise, int64_t* indices, float* weights,
+             void* workspace, size_t workspace_bytes, void* stream);
+
+/* lmk_score followed by lmk_topk; scores (N, C, E) is written and is an output too.
+ * Replaces model/DRT.py:612-627. */
+int lmk_score_topk(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, const void* noise,
+                   void* scores, int64_t* indices, float* weights,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GCA_HIP_H */

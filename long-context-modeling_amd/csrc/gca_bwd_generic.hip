@@ -1,0 +1,293 @@
+// Generic GCA backward: fp32 arithmetic on the vector ALUs for any supported shape and
+// element type (the fp32 path and the fallback for shapes the MFMA kernels do not take).
+//
+// Three launches, no atomics in the gathered form:
+//   1. dq kernel   one workgroup = 32 query rows of one (z, query head).  Per retrieved chunk
+//                  it makes two passes over the key tiles: the first builds
+//                  D_j = rowsum(P_j * dP_j) (stored to `delta`), the second forms
+//                  dS = w P (dP - D_j) and accumulates dQ += dS K.
+//   2. dkdv kernel one workgroup = 32 key rows of one (z, kv head, retrieved chunk); loops over
+//                  the query heads of the group and their rows, using lse and delta.
+//                  Gathered form: writes dk, dv in T.  Indexed form: atomically adds into the
+//                  float cache-shaped gradient buffers (several query chunks may have
+//                  retrieved the same cache chunk).
+//   3. dw kernel   dw[z, j] = sum over heads and rows of delta.
+// Same lane mapping as the generic forward: 8 lanes share a row and own D/8 dims each.
+#include "gca_common.h"
+
+namespace gca {
+
+template <typename T, typename WT, int D>
+__global__ void __launch_bounds__(256)
+gca_bwd_dq_generic_kernel(Params p, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+                          const int64_t* __restrict__ indices, const WT* __restrict__ w,
+                          const T* __restrict__ dout, const float* __restrict__ lse,
+                          T* __restrict__ dq, float* __restrict__ delta) {
+    constexpr int TPR = 8, QB = 32, DPT = D / TPR;
+    constexpr int KT = (D >= 256) ? 16 : 32;
+    __shared__ float sK[KT * D];
+    __shared__ float sV[KT * D];
+
+    const int tid = threadIdx.x;
+    const int r = tid / TPR, t = tid % TPR;
+    const int nqb = (p.Q_CTX + QB - 1) / QB;
+    const int64_t bid = blockIdx.x;
+    const int qb = (int)(bid % nqb);
+    const int64_t zh = bid / nqb;
+    const int h = (int)(zh % p.Hq);
+    const int64_t z = zh / p.Hq;
+    const int hk = h / p.G;
+    const int row = qb * QB + r;
+    const bool row_ok = row < p.Q_CTX;
+
+    float qreg[DPT], doreg[DPT], dqacc[DPT];
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) { qreg[i] = 0.f; doreg[i] = 0.f; dqacc[i] = 0.f; }
+    const int64_t qoff = ((z * p.Hq + h) * (int64_t)p.Q_CTX + row) * D + t * DPT;
+    if (row_ok) {
+#pragma unroll
+        for (int i = 0; i < DPT; ++i) { qreg[i] = to_f(q[qoff + i]); doreg[i] = to_f(dout[qoff + i]); }
+    }
+    const float c = p.sm_scale * LOG2E;
+
+    for (int j = 0; j < p.K; ++j) {
+        int64_t rs;
+        const T* kj = chunk_base(p, k, indices, z, hk, j, rs);
+        const T* vj = chunk_base(p, v, indices, z, hk, j, rs);
+        const int64_t loff = ((z * p.Hq + h) * (int64_t)p.K + j) * p.Q_CTX + row;
+        const float lse_r = row_ok ? lse[loff] : 0.f;
+        const float wj = to_f(w[z * p.K + j]);
+        float Dj = 0.f;
+        for (int pass = 0; pass < 2; ++pass) {
+            for (int kt0 = 0; kt0 < p.K_CTX; kt0 += KT) {
+                __syncthreads();
+                for (int i = tid; i < KT * D; i += 256) {
+                    const int key = i / D, dd = i % D;
+                    const int gk = kt0 + key;
+                    float kv = 0.f, vv = 0.f;
+                    if (gk < p.K_CTX) {
+                        kv = to_f(kj[(int64_t)gk * rs + dd]);
+                        vv = to_f(vj[(int64_t)gk * rs + dd]);
+                    }
+                    sK[i] = kv;
+                    sV[i] = vv;
+                }
+                __syncthreads();
+                const int nk = min(KT, p.K_CTX - kt0);
+#pragma unroll 4
+                for (int kk = 0; kk < KT; ++kk) {
+                    float s = 0.f, dp = 0.f;
+#pragma unroll
+                    for (int i = 0; i < DPT; ++i) {
+                        s = fmaf(qreg[i], sK[kk * D + t * DPT + i], s);
+                        dp = fmaf(doreg[i], sV[kk * D + t * DPT + i], dp);
+                    }
+                    s += __shfl_xor(s, 1);  dp += __shfl_xor(dp, 1);
+                    s += __shfl_xor(s, 2);  dp += __shfl_xor(dp, 2);
+                    s += __shfl_xor(s, 4);  dp += __shfl_xor(dp, 4);
+                    const float pe = (kk < nk) ? exp2f(s * c - lse_r) : 0.f;
+                    if (pass == 0) {
+                        Dj = fmaf(pe, dp, Dj);
+                    } else {
+                        const float ds = wj * pe * (dp - Dj);
+#pragma unroll
+                        for (int i = 0; i < DPT; ++i) dqacc[i] = fmaf(ds, sK[kk * D + t * DPT + i], dqacc[i]);
+                    }
+                }
+            }
+        }
+        if (row_ok && t == 0) delta[loff] = Dj;
+    }
+    if (row_ok) {
+#pragma unroll
+        for (int i = 0; i < DPT; ++i) dq[qoff + i] = from_f<T>(dqacc[i] * p.sm_scale);
+    }
+}
+
+template <typename T, typename WT, int D, bool INDEXED>
+__global__ void __launch_bounds__(256)
+gca_bwd_dkdv_generic_kernel(Params p, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+                            const int64_t* __restrict__ indices, const WT* __restrict__ w,
+                            const T* __restrict__ dout, const float* __restrict__ lse,
+                            const float* __restrict__ delta, void* __restrict__ dk_out, void* __restrict__ dv_out) {
+    constexpr int TPR = 8, KB = 32, DPT = D / TPR;
+    constexpr int QT = (D >= 256) ? 16 : 32;
+    __shared__ float sQ[QT * D];
+    __shared__ float sDO[QT * D];
+    __shared__ float sL[QT];
+    __shared__ float sDl[QT];
+
+    const int tid = threadIdx.x;
+    const int r = tid / TPR, t = tid % TPR;
+    const int nkb = (p.K_CTX + KB - 1) / KB;
+    int64_t bid = blockIdx.x;
+    const int kb = (int)(bid % nkb); bid /= nkb;
+    const int j = (int)(bid % p.K); bid /= p.K;
+    const int hk = (int)(bid % p.Hkv);
+    const int64_t z = bid / p.Hkv;
+    const int krow = kb * KB + r;
+    const bool row_ok = krow < p.K_CTX;
+
+    int64_t rs;
+    const T* kj = chunk_base(p, k, indices, z, hk, j, rs);
+    const T* vj = chunk_base(p, v, indices, z, hk, j, rs);
+    float kreg[DPT], vreg[DPT], dkacc[DPT], dvacc[DPT];
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) { kreg[i] = 0.f; vreg[i] = 0.f; dkacc[i] = 0.f; dvacc[i] = 0.f; }
+    if (row_ok) {
+#pragma unroll
+        for (int i = 0; i < DPT; ++i) {
+            kreg[i] = to_f(kj[(int64_t)krow * rs + t * DPT + i]);
+            vreg[i] = to_f(vj[(int64_t)krow * rs + t * DPT + i]);
+        }
+    }
+    const float c = p.sm_scale * LOG2E;
+    const float wj = to_f(w[z * p.K + j]);
+
+    for (int g = 0; g < p.G; ++g) {
+        const int h = hk * p.G + g;
+        const int64_t qbase = (z * p.Hq + h) * (int64_t)p.Q_CTX;
+        const int64_t lbase = ((z * p.Hq + h) * (int64_t)p.K + j) * p.Q_CTX;
+        for (int q0 = 0; q0 < p.Q_CTX; q0 += QT) {
+            __syncthreads();
+            for (int i = tid; i < QT * D; i += 256) {
+                const int qq = i / D, dd = i % D;
+                const int gq = q0 + qq;
+                float a = 0.f, b = 0.f;
+                if (gq < p.Q_CTX) {
+                    a = to_f(q[(qbase + gq) * D + dd]);
+                    b = to_f(dout[(qbase + gq) * D + dd]);
+                }
+                sQ[i] = a;
+                sDO[i] = b;
+            }
+            if (tid < QT) {
+                const int gq = q0 + tid;
+                sL[tid] = gq < p.Q_CTX ? lse[lbase + gq] : 0.f;
+                sDl[tid] = gq < p.Q_CTX ? delta[lbase + gq] : 0.f;
+            }
+            __syncthreads();
+            const int nq = min(QT, p.Q_CTX - q0);
+#pragma unroll 4
+            for (int qq = 0; qq < QT; ++qq) {
+                float s = 0.f, dp = 0.f;
+#pragma unroll
+                for (int i = 0; i < DPT; ++i) {
+                    s = fmaf(kreg[i], sQ[qq * D + t * DPT + i], s);
+                    dp = fmaf(vreg[i], sDO[qq * D + t * DPT + i], dp);
+                }
+                s += __shfl_xor(s, 1);  dp += __shfl_xor(dp, 1);
+                s += __shfl_xor(s, 2);  dp += __shfl_xor(dp, 2);
+                s += __shfl_xor(s, 4);  dp += __shfl_xor(dp, 4);
+                const float pw = (qq < nq) ? wj * exp2f(s * c - sL[qq]) : 0.f;
+                const float ds = pw * (dp - sDl[qq]);
+#pragma unroll
+                for (int i = 0; i < DPT; ++i) {
+                    dvacc[i] = fmaf(pw, sDO[qq * D + t * DPT + i], dvacc[i]);
+                    dkacc[i] = fmaf(ds, sQ[qq * D + t * DPT + i], dkacc[i]);
+                }
+            }
+        }
+    }
+    if (row_ok) {
+        if (INDEXED) {
+            const int64_t n = z / p.zpn;
+            int64_t cidx = indices[z * p.K + j];
+            cidx = cidx < 0 ? 0 : (cidx >= p.C ? p.C - 1 : cidx);
+            const int64_t off = (((n * p.C + cidx) * p.K_CTX + krow) * p.Hkv + hk) * (int64_t)D + t * DPT;
+            float* dkc = (float*)dk_out + off;
+            float* dvc = (float*)dv_out + off;
+#pragma unroll
+            for (int i = 0; i < DPT; ++i) {
+                atomicAdd(dkc + i, dkacc[i] * p.sm_scale);
+                atomicAdd(dvc + i, dvacc[i]);
+            }
+        } else {
+            const int64_t off = ((((z * p.Hkv + hk) * p.K + j) * (int64_t)p.K_CTX) + krow) * D + t * DPT;
+            T* dkp = (T*)dk_out + off;
+            T* dvp = (T*)dv_out + off;
+#pragma unroll
+            for (int i = 0; i < DPT; ++i) {
+                dkp[i] = from_f<T>(dkacc[i] * p.sm_scale);
+                dvp[i] = from_f<T>(dvacc[i]);
+            }
+        }
+    }
+}
+
+// dw[z, j] = sum_{h, m} delta[z, h, j, m]   (one wavefront per (z, j), fixed summation order)
+__global__ void __launch_bounds__(64)
+gca_bwd_dw_kernel(Params p, const float* __restrict__ delta, float* __restrict__ dw) {
+    const int64_t zj = blockIdx.x;
+    const int64_t z = zj / p.K;
+    const int j = (int)(zj % p.K);
+    float acc = 0.f;
+    const int total = p.Hq * p.Q_CTX;
+    for (int i = threadIdx.x; i < total; i += 64) {
+        const int h = i / p.Q_CTX, m = i % p.Q_CTX;
+        acc += delta[((z * p.Hq + h) * (int64_t)p.K + j) * p.Q_CTX + m];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+    if (threadIdx.x == 0) dw[zj] = acc;
+}
+
+int launch_dw(const Params& p, const float* delta, float* dw, hipStream_t s) {
+    const int64_t blocks = p.Z * p.K;
+    if (blocks <= 0 || blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
+    hipLaunchKernelGGL(gca_bwd_dw_kernel, dim3((unsigned)blocks), dim3(64), 0, s, p, delta, dw);
+    return hipGetLastError() == hipSuccess ? GCA_OK : GCA_ERR_LAUNCH;
+}
+
+template <typename T, typename WT, int D>
+static int launch_d(const Params& p, const void* q, const void* k, const void* v, const int64_t* idx,
+                    const void* w, const void* dout, const float* lse, void* dq, void* dk, void* dv,
+                    float* dw, float* delta, hipStream_t s) {
+    const int nqb = (p.Q_CTX + 31) / 32;
+    const int64_t b1 = p.Z * p.Hq * nqb;
+    const int nkb = (p.K_CTX + 31) / 32;
+    const int64_t b2 = p.Z * p.Hkv * p.K * nkb;
+    if (b1 <= 0 || b1 > 0x7fffffffLL || b2 <= 0 || b2 > 0x7fffffffLL) return GCA_ERR_SHAPE;
+    hipLaunchKernelGGL((gca_bwd_dq_generic_kernel<T, WT, D>), dim3((unsigned)b1), dim3(256), 0, s, p,
+                       (const T*)q, (const T*)k, (const T*)v, idx, (const WT*)w, (const T*)dout, lse, (T*)dq, delta);
+    if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
+    if (p.indexed)
+        hipLaunchKernelGGL((gca_bwd_dkdv_generic_kernel<T, WT, D, true>), dim3((unsigned)b2), dim3(256), 0, s, p,
+                           (const T*)q, (const T*)k, (const T*)v, idx, (const WT*)w, (const T*)dout, lse, delta, dk, dv);
+    else
+        hipLaunchKernelGGL((gca_bwd_dkdv_generic_kernel<T, WT, D, false>), dim3((unsigned)b2), dim3(256), 0, s, p,
+                           (const T*)q, (const T*)k, (const T*)v, idx, (const WT*)w, (const T*)dout, lse, delta, dk, dv);
+    if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
+    return launch_dw(p, delta, dw, s);
+}
+
+template <typename T, typename WT>
+static int launch_t(const Params& p, const void* q, const void* k, const void* v, const int64_t* idx,
+                    const void* w, const void* dout, const float* lse, void* dq, void* dk, void* dv,
+                    float* dw, float* delta, hipStream_t s) {
+    switch (p.D) {
+        case 16: return launch_d<T, WT, 16>(p, q, k, v, idx, w, dout, lse, dq, dk, dv, dw, delta, s);
+        case 32: return launch_d<T, WT, 32>(p, q, k, v, idx, w, dout, lse, dq, dk, dv, dw, delta, s);
+        case 64: return launch_d<T, WT, 64>(p, q, k, v, idx, w, dout, lse, dq, dk, dv, dw, delta, s);
+        case 128: return launch_d<T, WT, 128>(p, q, k, v, idx, w, dout, lse, dq, dk, dv, dw, delta, s);
+        case 256: return launch_d<T, WT, 256>(p, q, k, v, idx, w, dout, lse, dq, dk, dv, dw, delta, s);
+    }
+    return GCA_ERR_SHAPE;
+}
+
+int launch_bwd_generic(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v,
+                       const int64_t* indices, const void* w, const void* dout, const float* lse,
+                       void* dq, void* dk, void* dv, float* dw, float* delta, hipStream_t s) {
+    const Params p = make_params(d, indexed);
+    if (d.dtype == GCA_F32 && d.w_dtype == GCA_F32)
+        return launch_t<float, float>(p, q, k, v, indices, w, dout, lse, dq, dk, dv, dw, delta, s);
+    if (d.dtype == GCA_F32 && d.w_dtype == GCA_BF16)
+        return launch_t<float, bf16_t>(p, q, k, v, indices, w, dout, lse, dq, dk, dv, dw, delta, s);
+    if (d.dtype == GCA_BF16 && d.w_dtype == GCA_F32)
+        return launch_t<bf16_t, float>(p, q, k, v, indices, w, dout, lse, dq, dk, dv, dw, delta, s);
+    if (d.dtype == GCA_BF16 && d.w_dtype == GCA_BF16)
+        return launch_t<bf16_t, bf16_t>(p, q, k, v, indices, w, dout, lse, dq, dk, dv, dw, delta, s);
+    return GCA_ERR_DTYPE;
+}
+
+}  // namespace gca

@@ -1,0 +1,148 @@
+// extern "C" surface of libgca_hip.so: argument validation and dispatch only.
+#include "gca_common.h"
+
+using namespace gca;
+
+namespace {
+
+int check_desc(const gca_desc* d, bool indexed) {
+    if (d == nullptr) return GCA_ERR_NULL;
+    if (d->dtype != GCA_F32 && d->dtype != GCA_BF16) return GCA_ERR_DTYPE;
+    if (d->w_dtype != GCA_F32 && d->w_dtype != GCA_BF16) return GCA_ERR_DTYPE;
+    if (d->Z <= 0 || d->Hq <= 0 || d->Hkv <= 0 || d->K <= 0 || d->Q_CTX <= 0 || d->K_CTX <= 0) return GCA_ERR_SHAPE;
+    if (d->Hq % d->Hkv != 0) return GCA_ERR_SHAPE;
+    if (d->D != 16 && d->D != 32 && d->D != 64 && d->D != 128 && d->D != 256) return GCA_ERR_SHAPE;
+    if (!(d->sm_n >= 0.f)) return GCA_ERR_SHAPE;
+    if (d->path != GCA_PATH_AUTO && d->path != GCA_PATH_GENERIC && d->path != GCA_PATH_MFMA) return GCA_ERR_SHAPE;
+    if (indexed) {
+        if (d->N <= 0 || d->C <= 0 || d->Z % d->N != 0) return GCA_ERR_SHAPE;
+    }
+    return GCA_OK;
+}
+
+int check_lmk(const lmk_desc* d) {
+    if (d == nullptr) return GCA_ERR_NULL;
+    if (d->dtype != GCA_F32 && d->dtype != GCA_BF16) return GCA_ERR_DTYPE;
+    if (d->N <= 0 || d->C <= 0 || d->E <= 0 || d->Dm <= 0 || d->topk <= 0) return GCA_ERR_SHAPE;
+    if (d->causal && d->C > d->E) return GCA_ERR_SHAPE;
+    if (!(d->hidden_size > 0.f)) return GCA_ERR_SHAPE;
+    return GCA_OK;
+}
+
+// returns GCA_OK and sets use_mfma, or an error
+int pick_path(const gca_desc& d, bool& use_mfma) {
+    const bool ok = mfma_supported(d);
+    if (d.path == GCA_PATH_MFMA && !ok) return GCA_ERR_UNSUPPORTED;
+    use_mfma = (d.path != GCA_PATH_GENERIC) && ok;
+    return GCA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int gca_version(void) { return 100; }
+
+const char* gca_strerror(int status) {
+    switch (status) {
+        case GCA_OK: return "ok";
+        case GCA_ERR_NULL: return "a required pointer is NULL";
+        case GCA_ERR_SHAPE: return "bad shape or size";
+        case GCA_ERR_DTYPE: return "unknown element type";
+        case GCA_ERR_LAUNCH: return "HIP refused the kernel launch (is this a gfx950 GPU?)";
+        case GCA_ERR_WORKSPACE: return "workspace missing or too small";
+        case GCA_ERR_UNSUPPORTED: return "no kernel for this request";
+    }
+    return "unknown status";
+}
+
+int gca_fwd(const gca_desc* desc, const void* q, const void* k, const void* v, const void* weights,
+            void* o, float* lse, void* stream) {
+    int rc = check_desc(desc, false);
+    if (rc != GCA_OK) return rc;
+    if (!q || !k || !v || !weights || !o) return GCA_ERR_NULL;
+    bool use_mfma = false;
+    if ((rc = pick_path(*desc, use_mfma)) != GCA_OK) return rc;
+    if (use_mfma) return launch_fwd_mfma(*desc, false, q, k, v, nullptr, weights, o, lse, (hipStream_t)stream);
+    return launch_fwd_generic(*desc, false, q, k, v, nullptr, weights, o, lse, (hipStream_t)stream);
+}
+
+size_t gca_bwd_workspace_bytes(const gca_desc* desc) {
+    if (check_desc(desc, false) != GCA_OK) return 0;
+    return (size_t)desc->Z * desc->Hq * desc->K * desc->Q_CTX * sizeof(float);
+}
+
+int gca_bwd(const gca_desc* desc, const void* q, const void* k, const void* v, const void* weights,
+            const void* dout, const float* lse, void* dq, void* dk, void* dv, float* dw,
+            void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_desc(desc, false);
+    if (rc != GCA_OK) return rc;
+    if (!q || !k || !v || !weights || !dout || !lse || !dq || !dk || !dv || !dw) return GCA_ERR_NULL;
+    if (!workspace || workspace_bytes < gca_bwd_workspace_bytes(desc)) return GCA_ERR_WORKSPACE;
+    bool use_mfma = false;
+    if ((rc = pick_path(*desc, use_mfma)) != GCA_OK) return rc;
+    if (use_mfma)
+        return launch_bwd_mfma(*desc, false, q, k, v, nullptr, weights, dout, lse, dq, dk, dv, dw, (float*)workspace,
+                               (hipStream_t)stream);
+    return launch_bwd_generic(*desc, false, q, k, v, nullptr, weights, dout, lse, dq, dk, dv, dw, (float*)workspace,
+                              (hipStream_t)stream);
+}
+
+int gca_fwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, const void* v_cache,
+                    const int64_t* indices, const void* weights, void* o, float* lse, void* stream) {
+    int rc = check_desc(desc, true);
+    if (rc != GCA_OK) return rc;
+    if (!q || !k_cache || !v_cache || !indices || !weights || !o) return GCA_ERR_NULL;
+    bool use_mfma = false;
+    if ((rc = pick_path(*desc, use_mfma)) != GCA_OK) return rc;
+    if (use_mfma) return launch_fwd_mfma(*desc, true, q, k_cache, v_cache, indices, weights, o, lse, (hipStream_t)stream);
+    return launch_fwd_generic(*desc, true, q, k_cache, v_cache, indices, weights, o, lse, (hipStream_t)stream);
+}
+
+int gca_bwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, const void* v_cache,
+                    const int64_t* indices, const void* weights, const void* dout, const float* lse,
+                    void* dq, float* dk_cache, float* dv_cache, float* dw,
+                    void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_desc(desc, true);
+    if (rc != GCA_OK) return rc;
+    if (!q || !k_cache || !v_cache || !indices || !weights || !dout || !lse || !dq || !dk_cache || !dv_cache || !dw)
+        return GCA_ERR_NULL;
+    if (!workspace || workspace_bytes < gca_bwd_workspace_bytes(desc)) return GCA_ERR_WORKSPACE;
+    bool use_mfma = false;
+    if ((rc = pick_path(*desc, use_mfma)) != GCA_OK) return rc;
+    if (use_mfma)
+        return launch_bwd_mfma(*desc, true, q, k_cache, v_cache, indices, weights, dout, lse, dq, dk_cache, dv_cache, dw,
+                               (float*)workspace, (hipStream_t)stream);
+    return launch_bwd_generic(*desc, true, q, k_cache, v_cache, indices, weights, dout, lse, dq, dk_cache, dv_cache, dw,
+                              (float*)workspace, (hipStream_t)stream);
+}
+
+int lmk_score(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, void* scores, void* stream) {
+    int rc = check_lmk(desc);
+    if (rc != GCA_OK) return rc;
+    if (!lmk_q || !lmk_k || !scores) return GCA_ERR_NULL;
+    return launch_lmk_score(*desc, lmk_q, lmk_k, scores, (hipStream_t)stream);
+}
+
+size_t lmk_topk_workspace_bytes(const lmk_desc* desc) {
+    if (check_lmk(desc) != GCA_OK) return 0;
+    return lmk_topk_ws_bytes(*desc);
+}
+
+int lmk_topk(const lmk_desc* desc, const void* scores, const void* noise, int64_t* indices, float* weights,
+             void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_lmk(desc);
+    if (rc != GCA_OK) return rc;
+    if (!scores || !indices || !weights) return GCA_ERR_NULL;
+    return launch_lmk_topk(*desc, scores, noise, indices, weights, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+int lmk_score_topk(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, const void* noise,
+                   void* scores, int64_t* indices, float* weights,
+                   void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = lmk_score(desc, lmk_q, lmk_k, scores, stream);
+    if (rc != GCA_OK) return rc;
+    return lmk_topk(desc, scores, noise, indices, weights, workspace, workspace_bytes, stream);
+}
+
+}  // extern "C"

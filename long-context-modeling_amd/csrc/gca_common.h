@@ -1,0 +1,89 @@
+// Shared device/host helpers for the GCA kernels (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "gca_hip.h"
+
+namespace gca {
+
+constexpr float LOG2E = 1.4426950408889634f;
+
+// bf16 stored as raw 16 bits; conversion is a shift, rounding is nearest-even.
+struct bf16_t {
+    uint16_t x;
+};
+
+__device__ __forceinline__ float bf16_bits_to_f(uint32_t bits) { return __uint_as_float(bits << 16); }
+
+__device__ __forceinline__ uint16_t f_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);  // NaN stays NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float to_f(float v) { return v; }
+__device__ __forceinline__ float to_f(bf16_t v) { return bf16_bits_to_f(v.x); }
+
+template <typename T> __device__ __forceinline__ T from_f(float f);
+template <> __device__ __forceinline__ float from_f<float>(float f) { return f; }
+template <> __device__ __forceinline__ bf16_t from_f<bf16_t>(float f) { return bf16_t{f_to_bf16_bits(f)}; }
+
+// Plain-old-data copy of the descriptor plus derived values, passed by value to kernels.
+struct Params {
+    int64_t Z;
+    int32_t Hq, Hkv, G, K, Q_CTX, K_CTX, D;
+    float sm_scale, sm_n;
+    // indexed variants
+    int64_t N, C, zpn;   // zpn = Z / N rows per sequence
+    int32_t indexed;
+};
+
+inline Params make_params(const gca_desc& d, bool indexed) {
+    Params p;
+    p.Z = d.Z; p.Hq = d.Hq; p.Hkv = d.Hkv; p.G = d.Hq / d.Hkv; p.K = d.K;
+    p.Q_CTX = d.Q_CTX; p.K_CTX = d.K_CTX; p.D = d.D;
+    p.sm_scale = d.sm_scale; p.sm_n = d.sm_n;
+    p.N = indexed ? d.N : 1; p.C = indexed ? d.C : 1;
+    p.zpn = indexed ? d.Z / d.N : d.Z;
+    p.indexed = indexed ? 1 : 0;
+    return p;
+}
+
+// Address of element (key row 0, dim 0) of retrieved chunk j for row z, kv head hk, and the
+// distance in elements between consecutive key rows.  Gathered form: k is (Z,Hkv,K,K_CTX,D);
+// indexed form: cache is (N,C,K_CTX,Hkv*D) and the chunk id comes from indices[z,j].
+template <typename T>
+__device__ __forceinline__ const T* chunk_base(const Params& p, const T* base, const int64_t* indices,
+                                               int64_t z, int hk, int j, int64_t& row_stride) {
+    if (p.indexed) {
+        const int64_t n = z / p.zpn;
+        int64_t c = indices[z * p.K + j];
+        c = c < 0 ? 0 : (c >= p.C ? p.C - 1 : c);   // out-of-range ids never leave the cache
+        row_stride = (int64_t)p.Hkv * p.D;
+        return base + ((n * p.C + c) * p.K_CTX) * row_stride + (int64_t)hk * p.D;
+    }
+    row_stride = p.D;
+    return base + (((z * p.Hkv + hk) * p.K + j) * (int64_t)p.K_CTX) * p.D;
+}
+
+}  // namespace gca
+
+// Launchers implemented in the kernel translation units; all return a gca_status.
+namespace gca {
+int launch_fwd_generic(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v,
+                       const int64_t* indices, const void* w, void* o, float* lse, hipStream_t s);
+int launch_bwd_generic(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v,
+                       const int64_t* indices, const void* w, const void* dout, const float* lse,
+                       void* dq, void* dk, void* dv, float* dw, float* delta, hipStream_t s);
+bool mfma_supported(const gca_desc& d);
+int launch_fwd_mfma(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v,
+                    const int64_t* indices, const void* w, void* o, float* lse, hipStream_t s);
+int launch_bwd_mfma(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v,
+                    const int64_t* indices, const void* w, const void* dout, const float* lse,
+                    void* dq, void* dk, void* dv, float* dw, float* delta, hipStream_t s);
+int launch_lmk_score(const lmk_desc& d, const void* lq, const void* lk, void* scores, hipStream_t s);
+int launch_lmk_topk(const lmk_desc& d, const void* scores, const void* noise, int64_t* indices, float* weights,
+                    void* ws, size_t ws_bytes, hipStream_t s);
+size_t lmk_topk_ws_bytes(const lmk_desc& d);
+}  // namespace gca

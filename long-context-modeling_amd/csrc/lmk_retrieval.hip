@@ -1,0 +1,410 @@
+// Landmark retrieval: scoring, strict-past mask, top-k selection, retrieval weights.
+//
+//   lmk_score   two kernels.  "scan": few query rows per sequence (decode): one wavefront per
+//               candidate landmark, 16-byte loads, wavefront reduction -- an HBM-bound stream
+//               over lmk_k.  "tile": many query rows (training/prefill): 32x32 output tiles,
+//               operands staged through LDS, tiles that are entirely masked are only filled.
+//   lmk_topk    bitonic top-k in LDS over 64-bit keys (order-preserving image of the float in
+//               the high half, inverted index in the low half), so "higher value first, then
+//               lower index" is one unsigned compare and the result is unique.  Long rows are
+//               cut into segments (one workgroup each) whose winners a second launch merges.
+#include "gca_common.h"
+
+namespace gca {
+
+// ------------------------------------------------------------------------------------ scoring
+
+template <typename T> struct Vec16;   // 16-byte vector of T
+template <> struct Vec16<float> { static constexpr int N = 4; };
+template <> struct Vec16<bf16_t> { static constexpr int N = 8; };
+
+template <typename T>
+__device__ __forceinline__ float finish_score(float dot, float sqrt_hidden);
+template <> __device__ __forceinline__ float finish_score<float>(float dot, float sqrt_hidden) { return dot / sqrt_hidden; }
+// bf16: the product is rounded to bf16, then the division result is rounded again
+// (a bf16 matmul followed by a bf16 division).
+template <> __device__ __forceinline__ float finish_score<bf16_t>(float dot, float sqrt_hidden) {
+    const float r1 = bf16_bits_to_f(f_to_bf16_bits(dot));
+    return bf16_bits_to_f(f_to_bf16_bits(r1 / sqrt_hidden));
+}
+
+__device__ __forceinline__ void unpack16(const uint4& raw, float (&out)[8]) {
+    const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        out[2 * i] = __uint_as_float(u[i] << 16);
+        out[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
+    }
+}
+
+// One wavefront per candidate landmark e; all C (<= SCAN_MAX_C) query rows of the sequence
+// sit in LDS as floats.  Requires Dm % (16 / sizeof(T)) == 0.
+constexpr int SCAN_MAX_C = 4;
+constexpr int SCAN_EPW = 4;   // landmarks per wavefront per iteration (loads issued together)
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+lmk_score_scan_kernel(lmk_desc d, const T* __restrict__ lq, const T* __restrict__ lk, T* __restrict__ scores) {
+    constexpr int VN = Vec16<T>::N;
+    extern __shared__ float sq[];   // C * Dm
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t n = blockIdx.y;
+    const int C = (int)d.C, Dm = d.Dm;
+    for (int i = tid; i < C * Dm; i += 256) sq[i] = to_f(lq[n * C * Dm + i]);
+    __syncthreads();
+    const float sqrt_hidden = sqrtf(d.hidden_size);
+    const int nvec = Dm / VN;
+    const int64_t e0 = ((int64_t)blockIdx.x * 4 + wave) * SCAN_EPW;
+    float acc[SCAN_EPW][SCAN_MAX_C];
+#pragma unroll
+    for (int a = 0; a < SCAN_EPW; ++a)
+#pragma unroll
+        for (int c = 0; c < SCAN_MAX_C; ++c) acc[a][c] = 0.f;
+
+    for (int iv = lane; iv < nvec; iv += 64) {
+        uint4 raw[SCAN_EPW];
+#pragma unroll
+        for (int a = 0; a < SCAN_EPW; ++a) {
+            const int64_t e = e0 + a;
+            raw[a] = make_uint4(0, 0, 0, 0);
+            if (e < d.E) raw[a] = *reinterpret_cast<const uint4*>(lk + (n * d.E + e) * Dm + (int64_t)iv * VN);
+        }
+#pragma unroll
+        for (int a = 0; a < SCAN_EPW; ++a) {
+            float kv[8];
+            if (VN == 8) {
+                unpack16(raw[a], kv);
+            } else {
+                kv[0] = __uint_as_float(raw[a].x); kv[1] = __uint_as_float(raw[a].y);
+                kv[2] = __uint_as_float(raw[a].z); kv[3] = __uint_as_float(raw[a].w);
+            }
+#pragma unroll
+            for (int c = 0; c < SCAN_MAX_C; ++c) {
+                if (c < C) {
+#pragma unroll
+                    for (int i = 0; i < VN; ++i) acc[a][c] = fmaf(sq[c * Dm + iv * VN + i], kv[i], acc[a][c]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < SCAN_EPW; ++a) {
+#pragma unroll
+        for (int c = 0; c < SCAN_MAX_C; ++c) {
+            float x = acc[a][c];
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off);
+            const int64_t e = e0 + a;
+            if (lane == 0 && c < C && e < d.E) {
+                float r = finish_score<T>(x, sqrt_hidden);
+                if (d.causal && !((d.E - C + c) > e)) r = -INFINITY;
+                scores[(n * C + c) * d.E + e] = from_f<T>(r);
+            }
+        }
+    }
+}
+
+// 32x32 output tile per workgroup, 2x2 outputs per thread, Dm consumed in steps of 32.
+template <typename T>
+__global__ void __launch_bounds__(256)
+lmk_score_tile_kernel(lmk_desc d, const T* __restrict__ lq, const T* __restrict__ lk, T* __restrict__ scores) {
+    __shared__ float sA[32][33];
+    __shared__ float sB[32][33];
+    const int tid = threadIdx.x;
+    const int tx = tid & 15, ty = tid >> 4;
+    const int64_t n = blockIdx.z;
+    const int64_t c0 = (int64_t)blockIdx.y * 32, e0 = (int64_t)blockIdx.x * 32;
+    const int64_t off = d.E - d.C;
+    const int64_t cmax = min(c0 + 31, d.C - 1);
+    const bool all_masked = d.causal && !((off + cmax) > e0);
+    float acc[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+    if (!all_masked) {
+        for (int k0 = 0; k0 < d.Dm; k0 += 32) {
+            __syncthreads();
+            for (int i = tid; i < 1024; i += 256) {
+                const int rr = i >> 5, kk = i & 31;
+                const bool kin = (k0 + kk) < d.Dm;
+                sA[rr][kk] = (kin && (c0 + rr) < d.C) ? to_f(lq[(n * d.C + c0 + rr) * d.Dm + k0 + kk]) : 0.f;
+                sB[rr][kk] = (kin && (e0 + rr) < d.E) ? to_f(lk[(n * d.E + e0 + rr) * d.Dm + k0 + kk]) : 0.f;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int kk = 0; kk < 32; ++kk) {
+                const float a0 = sA[ty * 2][kk], a1 = sA[ty * 2 + 1][kk];
+                const float b0 = sB[tx * 2][kk], b1 = sB[tx * 2 + 1][kk];
+                acc[0][0] = fmaf(a0, b0, acc[0][0]);
+                acc[0][1] = fmaf(a0, b1, acc[0][1]);
+                acc[1][0] = fmaf(a1, b0, acc[1][0]);
+                acc[1][1] = fmaf(a1, b1, acc[1][1]);
+            }
+        }
+    }
+    const float sqrt_hidden = sqrtf(d.hidden_size);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int jx = 0; jx < 2; ++jx) {
+            const int64_t c = c0 + ty * 2 + i, e = e0 + tx * 2 + jx;
+            if (c < d.C && e < d.E) {
+                float r = finish_score<T>(acc[i][jx], sqrt_hidden);
+                if (d.causal && !((off + c) > e)) r = -INFINITY;
+                scores[(n * d.C + c) * d.E + e] = from_f<T>(r);
+            }
+        }
+}
+
+template <typename T>
+static int launch_score_t(const lmk_desc& d, const void* lq, const void* lk, void* scores, hipStream_t s) {
+    constexpr int VN = Vec16<T>::N;
+    const bool aligned = (((uintptr_t)lk) % 16 == 0) && (d.Dm % VN == 0);
+    const size_t lds = (size_t)d.C * d.Dm * sizeof(float);
+    if (d.C <= SCAN_MAX_C && aligned && lds <= 48 * 1024 && d.N <= 65535) {
+        const int64_t per_block = 4 * SCAN_EPW;
+        const int64_t bx = (d.E + per_block - 1) / per_block;
+        if (bx > 0x7fffffffLL) return GCA_ERR_SHAPE;
+        hipLaunchKernelGGL((lmk_score_scan_kernel<T>), dim3((unsigned)bx, (unsigned)d.N), dim3(256), lds, s, d,
+                           (const T*)lq, (const T*)lk, (T*)scores);
+    } else {
+        const int64_t bx = (d.E + 31) / 32, by = (d.C + 31) / 32;
+        if (bx > 0x7fffffffLL || by > 65535 || d.N > 65535) return GCA_ERR_SHAPE;
+        hipLaunchKernelGGL((lmk_score_tile_kernel<T>), dim3((unsigned)bx, (unsigned)by, (unsigned)d.N), dim3(256), 0, s, d,
+                           (const T*)lq, (const T*)lk, (T*)scores);
+    }
+    return hipGetLastError() == hipSuccess ? GCA_OK : GCA_ERR_LAUNCH;
+}
+
+int launch_lmk_score(const lmk_desc& d, const void* lq, const void* lk, void* scores, hipStream_t s) {
+    if (d.dtype == GCA_F32) return launch_score_t<float>(d, lq, lk, scores, s);
+    if (d.dtype == GCA_BF16) return launch_score_t<bf16_t>(d, lq, lk, scores, s);
+    return GCA_ERR_DTYPE;
+}
+
+// ------------------------------------------------------------------------------------ top-k
+
+constexpr int TOPK_TILE = 2048;      // keys per LDS tile
+constexpr int TOPK_THREADS = 256;
+constexpr int TOPK_MAX_KP = 128;     // largest supported power-of-two k
+
+__device__ __forceinline__ uint32_t sortable_bits(float v) {
+    if (v != v) return 0xffffffffu;                 // NaN ranks above everything, as in torch.topk
+    uint32_t u = (v == 0.f) ? 0u : __float_as_uint(v);   // -0 and +0 tie
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ uint64_t make_key(float v, uint32_t idx) {
+    return ((uint64_t)sortable_bits(v) << 32) | (uint64_t)(0xffffffffu - idx);
+}
+__device__ __forceinline__ uint32_t key_index(uint64_t key) { return 0xffffffffu - (uint32_t)(key & 0xffffffffu); }
+
+__device__ __forceinline__ void cmpx(uint64_t* keys, int lo, int hi, bool desc) {
+    const uint64_t a = keys[lo], b = keys[hi];
+    if ((a < b) == desc) { keys[lo] = b; keys[hi] = a; }
+}
+
+// Leaves the kp largest of keys[0, TOPK_TILE) in keys[0, kp), sorted descending.
+// kp is a power of two <= TOPK_MAX_KP.  All TOPK_THREADS threads of the workgroup must call it.
+__device__ void block_topk(uint64_t* keys, int kp, int tid) {
+    // sort groups of kp; even groups descending, odd groups ascending
+    for (int size = 2; size <= kp; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            for (int i = tid; i < TOPK_TILE / 2; i += TOPK_THREADS) {
+                const int lo = (i / stride) * 2 * stride + (i % stride);
+                cmpx(keys, lo, lo + stride, (lo & size) == 0);
+            }
+        }
+    }
+    // halve: (descending group, ascending group) is bitonic; the element-wise maximum keeps the
+    // kp largest as a bitonic sequence, which one merge pass sorts again
+    for (int n = TOPK_TILE; n > kp; n >>= 1) {
+        __syncthreads();
+        constexpr int PER = TOPK_TILE / 2 / TOPK_THREADS;
+        uint64_t tmp[PER];
+        const int half = n >> 1;
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int i = tid + u * TOPK_THREADS;
+            if (i < half) {
+                const int g = i / kp, r = i % kp;
+                const uint64_t a = keys[(2 * g) * kp + r], b = keys[(2 * g + 1) * kp + r];
+                tmp[u] = a > b ? a : b;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int i = tid + u * TOPK_THREADS;
+            if (i < half) keys[i] = tmp[u];
+        }
+        for (int stride = kp >> 1; stride > 0; stride >>= 1) {
+            __syncthreads();
+            for (int i = tid; i < half / 2; i += TOPK_THREADS) {
+                const int lo = (i / stride) * 2 * stride + (i % stride);
+                cmpx(keys, lo, lo + stride, (lo & kp) == 0);
+            }
+        }
+    }
+    __syncthreads();
+}
+
+template <typename T>
+__device__ __forceinline__ float round_like(float x);
+template <> __device__ __forceinline__ float round_like<float>(float x) { return x; }
+template <> __device__ __forceinline__ float round_like<bf16_t>(float x) { return bf16_bits_to_f(f_to_bf16_bits(x)); }
+
+// softmax over the kk selected noise-free masked scores; NaN (all -inf) -> 0
+template <typename T>
+__device__ void emit_row(const lmk_desc& d, const uint64_t* keys, int kk, int64_t row, int64_t limit,
+                         const T* __restrict__ scores, int64_t* __restrict__ indices, float* __restrict__ weights,
+                         float* sval, int tid) {
+    if (tid < kk) {
+        const uint32_t e = key_index(keys[tid]);
+        float sc = to_f(scores[row * d.E + e]);
+        if (d.causal && !((int64_t)e < limit)) sc = -INFINITY;
+        sval[tid] = sc;
+        indices[row * kk + tid] = (int64_t)e;
+    }
+    __syncthreads();
+    if (tid < kk) {
+        float m = -INFINITY;
+        for (int i = 0; i < kk; ++i) m = fmaxf(m, sval[i]);
+        float sum = 0.f;
+        for (int i = 0; i < kk; ++i) sum += expf(sval[i] - m);
+        float wv = expf(sval[tid] - m) / sum;
+        if (wv != wv) wv = 0.f;
+        weights[row * kk + tid] = wv;
+    }
+}
+
+// grid (nseg, R).  Segment `seg` of row `row` covers candidates [seg*seg_len, (seg+1)*seg_len)
+// clipped to the part of the row that can be selected.  nseg == 1 writes the final result,
+// otherwise the kp winners of the segment go to ws[(row*nseg + seg)*kp ...].
+template <typename T>
+__global__ void __launch_bounds__(TOPK_THREADS)
+lmk_topk_kernel(lmk_desc d, int kk, int kp, int nseg, int64_t seg_len, int64_t row0, const T* __restrict__ scores,
+                const T* __restrict__ noise, int64_t* __restrict__ indices, float* __restrict__ weights,
+                uint64_t* __restrict__ ws) {
+    __shared__ uint64_t keys[TOPK_TILE];
+    __shared__ float sval[TOPK_MAX_KP];
+    const int tid = threadIdx.x;
+    const int seg = blockIdx.x;
+    const int64_t row = row0 + blockIdx.y;
+    const int64_t c = row % d.C;
+    const int64_t limit = d.causal ? (d.E - d.C + c) : d.E;      // candidates e < limit are visible
+    // masked candidates all tie at -inf and rank by index, so only the first kk of the row matter
+    const int64_t scan_end = min(d.E, max(limit, (int64_t)kk));
+    const int64_t lo = (int64_t)seg * seg_len;
+    const int64_t hi = min(lo + seg_len, scan_end);
+
+    int carry = 0;   // keys[0, carry) hold the running winners
+    int64_t pos = lo;
+    do {
+        const int64_t take = TOPK_TILE - carry;
+        for (int i = tid; i < take; i += TOPK_THREADS) {
+            const int64_t e = pos + i;
+            uint64_t key = 0;
+            if (e < hi) {
+                float sv = to_f(scores[row * d.E + e]);
+                if (noise != nullptr) sv = round_like<T>(sv + to_f(noise[row * d.E + e]));
+                if (d.causal && !(e < limit)) sv = -INFINITY;
+                key = make_key(sv, (uint32_t)e);
+            }
+            keys[carry + i] = key;
+        }
+        block_topk(keys, kp, tid);
+        carry = kp;
+        pos += take;
+    } while (pos < hi);
+
+    if (nseg == 1) {
+        emit_row<T>(d, keys, kk, row, limit, scores, indices, weights, sval, tid);
+    } else if (tid < kp) {
+        ws[(row * nseg + seg) * kp + tid] = keys[tid];
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(TOPK_THREADS)
+lmk_topk_merge_kernel(lmk_desc d, int kk, int kp, int nseg, int64_t row0, const T* __restrict__ scores,
+                      int64_t* __restrict__ indices, float* __restrict__ weights, const uint64_t* __restrict__ ws) {
+    __shared__ uint64_t keys[TOPK_TILE];
+    __shared__ float sval[TOPK_MAX_KP];
+    const int tid = threadIdx.x;
+    const int64_t row = row0 + blockIdx.x;
+    const int64_t c = row % d.C;
+    const int64_t limit = d.causal ? (d.E - d.C + c) : d.E;
+    const int64_t total = (int64_t)nseg * kp;
+    int carry = 0;
+    int64_t pos = 0;
+    do {
+        const int64_t take = TOPK_TILE - carry;
+        for (int i = tid; i < take; i += TOPK_THREADS) {
+            const int64_t e = pos + i;
+            keys[carry + i] = e < total ? ws[row * total + e] : 0;
+        }
+        block_topk(keys, kp, tid);
+        carry = kp;
+        pos += take;
+    } while (pos < total);
+    emit_row<T>(d, keys, kk, row, limit, scores, indices, weights, sval, tid);
+}
+
+static int next_pow2(int x) { int p = 1; while (p < x) p <<= 1; return p; }
+
+struct TopkPlan { int kk, kp, nseg; int64_t seg_len; };
+
+static TopkPlan plan_topk(const lmk_desc& d) {
+    TopkPlan pl;
+    pl.kk = (int)((int64_t)d.topk < d.E ? d.topk : d.E);
+    pl.kp = next_pow2(pl.kk);
+    const int64_t R = d.N * d.C;
+    const int64_t tiles = (d.E + TOPK_TILE - 1) / TOPK_TILE;
+    int64_t want = (2048 + R - 1) / R;          // aim at >= 2048 workgroups
+    if (want < 1) want = 1;
+    if (want > tiles) want = tiles;
+    if (want > 1024) want = 1024;
+    pl.seg_len = ((d.E + want - 1) / want + TOPK_TILE - 1) / TOPK_TILE * TOPK_TILE;
+    pl.nseg = (int)((d.E + pl.seg_len - 1) / pl.seg_len);
+    return pl;
+}
+
+size_t lmk_topk_ws_bytes(const lmk_desc& d) {
+    if (d.E <= 0 || d.N <= 0 || d.C <= 0 || d.topk <= 0) return 0;
+    const TopkPlan pl = plan_topk(d);
+    return pl.nseg > 1 ? (size_t)(d.N * d.C) * pl.nseg * pl.kp * sizeof(uint64_t) : 0;
+}
+
+template <typename T>
+static int launch_topk_t(const lmk_desc& d, const TopkPlan& pl, const void* scores, const void* noise,
+                         int64_t* indices, float* weights, void* ws, hipStream_t s) {
+    // rows go in grid.y (at most 65535 per launch); rows are independent, so long inputs
+    // are cut into slabs and each launch is told its first row
+    const int64_t R = d.N * d.C;
+    const int64_t slab = 65535;
+    for (int64_t r0 = 0; r0 < R; r0 += slab) {
+        const int64_t rows = (R - r0) < slab ? (R - r0) : slab;
+        hipLaunchKernelGGL((lmk_topk_kernel<T>), dim3((unsigned)pl.nseg, (unsigned)rows), dim3(TOPK_THREADS), 0, s, d,
+                           pl.kk, pl.kp, pl.nseg, pl.seg_len, r0, (const T*)scores, (const T*)noise, indices, weights,
+                           (uint64_t*)ws);
+        if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
+        if (pl.nseg > 1) {
+            hipLaunchKernelGGL((lmk_topk_merge_kernel<T>), dim3((unsigned)rows), dim3(TOPK_THREADS), 0, s, d, pl.kk, pl.kp,
+                               pl.nseg, r0, (const T*)scores, indices, weights, (const uint64_t*)ws);
+            if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
+        }
+    }
+    return GCA_OK;
+}
+
+int launch_lmk_topk(const lmk_desc& d, const void* scores, const void* noise, int64_t* indices, float* weights,
+                    void* ws, size_t ws_bytes, hipStream_t s) {
+    const TopkPlan pl = plan_topk(d);
+    if (pl.kp > TOPK_MAX_KP) return GCA_ERR_UNSUPPORTED;
+    if (d.E > 0xffffffffLL) return GCA_ERR_SHAPE;
+    const size_t need = lmk_topk_ws_bytes(d);
+    if (need > 0 && (ws == nullptr || ws_bytes < need)) return GCA_ERR_WORKSPACE;
+    if (d.dtype == GCA_F32) return launch_topk_t<float>(d, pl, scores, noise, indices, weights, ws, s);
+    if (d.dtype == GCA_BF16) return launch_topk_t<bf16_t>(d, pl, scores, noise, indices, weights, ws, s);
+    return GCA_ERR_DTYPE;
+}
+
+}  // namespace gca

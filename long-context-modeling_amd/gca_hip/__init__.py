@@ -1,0 +1,9 @@
+"""MI355X-native Grouped Cross-Attention and landmark retrieval (HIP kernels behind a C ABI)."""
+from . import _lib
+from .gca import attention, gca_kv_cache, attention_indexed, gca_kv_cache_indexed
+from .retrieval import landmark_scores, landmark_topk, landmark_retrieve, gather_chunks, gca_layer
+
+__all__ = [
+    "attention", "gca_kv_cache", "attention_indexed", "gca_kv_cache_indexed",
+    "landmark_scores", "landmark_topk", "landmark_retrieve", "gather_chunks", "gca_layer",
+]

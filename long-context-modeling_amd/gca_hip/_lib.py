@@ -1,0 +1,96 @@
+"""ctypes binding of libgca_hip.so (declarations: include/gca_hip.h).
+
+There is no CPU fallback: if the library is missing or a call fails, callers get a
+RuntimeError / AssertionError.  Build it with ``make -C long-context-modeling_amd/csrc``
+(or ``python -c "import __graft_entry__ as g; g.build()"`` from the repository root).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libgca_hip.so")
+
+GCA_F32, GCA_BF16 = 0, 1
+GCA_PATH_AUTO, GCA_PATH_GENERIC, GCA_PATH_MFMA = 0, 1, 2
+GCA_OK = 0
+
+SYMBOLS = (
+    "gca_version", "gca_strerror", "gca_fwd", "gca_bwd_workspace_bytes", "gca_bwd", "gca_fwd_indexed",
+    "gca_bwd_indexed", "lmk_score", "lmk_topk_workspace_bytes", "lmk_topk", "lmk_score_topk",
+)
+
+
+class GcaDesc(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int32), ("w_dtype", ctypes.c_int32), ("Z", ctypes.c_int64),
+        ("Hq", ctypes.c_int32), ("Hkv", ctypes.c_int32), ("K", ctypes.c_int32),
+        ("Q_CTX", ctypes.c_int32), ("K_CTX", ctypes.c_int32), ("D", ctypes.c_int32),
+        ("sm_scale", ctypes.c_float), ("sm_n", ctypes.c_float),
+        ("path", ctypes.c_int32), ("reserved", ctypes.c_int32),
+        ("N", ctypes.c_int64), ("C", ctypes.c_int64),
+    ]
+
+
+class LmkDesc(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int32), ("topk", ctypes.c_int32),
+        ("N", ctypes.c_int64), ("C", ctypes.c_int64), ("E", ctypes.c_int64),
+        ("Dm", ctypes.c_int32), ("causal", ctypes.c_int32),
+        ("hidden_size", ctypes.c_float), ("reserved", ctypes.c_int32),
+    ]
+
+
+_lib = None
+_lock = threading.Lock()
+
+
+def _declare(lib):
+    P, I64P, FP = ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p
+    D, L = ctypes.POINTER(GcaDesc), ctypes.POINTER(LmkDesc)
+    lib.gca_version.restype = ctypes.c_int
+    lib.gca_version.argtypes = []
+    lib.gca_strerror.restype = ctypes.c_char_p
+    lib.gca_strerror.argtypes = [ctypes.c_int]
+    lib.gca_fwd.restype = ctypes.c_int
+    lib.gca_fwd.argtypes = [D, P, P, P, P, P, FP, P]
+    lib.gca_bwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.gca_bwd_workspace_bytes.argtypes = [D]
+    lib.gca_bwd.restype = ctypes.c_int
+    lib.gca_bwd.argtypes = [D, P, P, P, P, P, FP, P, P, P, FP, P, ctypes.c_size_t, P]
+    lib.gca_fwd_indexed.restype = ctypes.c_int
+    lib.gca_fwd_indexed.argtypes = [D, P, P, P, I64P, P, P, FP, P]
+    lib.gca_bwd_indexed.restype = ctypes.c_int
+    lib.gca_bwd_indexed.argtypes = [D, P, P, P, I64P, P, P, FP, P, FP, FP, FP, P, ctypes.c_size_t, P]
+    lib.lmk_score.restype = ctypes.c_int
+    lib.lmk_score.argtypes = [L, P, P, P, P]
+    lib.lmk_topk_workspace_bytes.restype = ctypes.c_size_t
+    lib.lmk_topk_workspace_bytes.argtypes = [L]
+    lib.lmk_topk.restype = ctypes.c_int
+    lib.lmk_topk.argtypes = [L, P, P, I64P, FP, P, ctypes.c_size_t, P]
+    lib.lmk_score_topk.restype = ctypes.c_int
+    lib.lmk_score_topk.argtypes = [L, P, P, P, P, I64P, FP, P, ctypes.c_size_t, P]
+
+
+def lib():
+    """The loaded library; raises RuntimeError when it has not been built."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                if not os.path.exists(LIB_PATH):
+                    raise RuntimeError(
+                        f"{LIB_PATH} is missing: the HIP kernels are not built and there is no fallback. "
+                        "Run `make -C long-context-modeling_amd/csrc`.")
+                handle = ctypes.CDLL(LIB_PATH)
+                _declare(handle)
+                _lib = handle
+    return _lib
+
+
+def check(status: int, what: str):
+    if status != GCA_OK:
+        msg = lib().gca_strerror(status).decode()
+        raise RuntimeError(f"{what} failed: {msg} (status {status})")

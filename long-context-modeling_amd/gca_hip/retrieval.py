@@ -1,0 +1,105 @@
+"""Landmark retrieval on MI355X: host side of the scoring / top-k kernels.
+
+Mirrors ``DRT._perform_batch_retrieval`` of the reference (model/DRT.py:609-641):
+score -> strict-past mask -> (noise) -> top-k -> softmax weights -> gather + kernel layout.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+
+import torch
+
+from . import _lib
+from .gca import _DT, _ptr, _stream
+
+
+def _lmk_desc(dtype, topk, N, C, E, Dm, causal, hidden_size):
+    return _lib.LmkDesc(dtype=_DT[dtype], topk=int(topk), N=N, C=C, E=E, Dm=Dm, causal=1 if causal else 0,
+                        hidden_size=float(hidden_size), reserved=0)
+
+
+def landmark_scores(lmk_q, lmk_k, hidden_size=None, causal=True):
+    """scores[n,c,e] = <lmk_q[n,c], lmk_k[n,e]> / sqrt(hidden), -inf where not strictly past
+    (model/DRT.py:612-613)."""
+    assert lmk_q.is_cuda and lmk_q.dim() == 3 and lmk_k.dim() == 3 and lmk_q.dtype in _DT and lmk_k.dtype == lmk_q.dtype
+    lmk_q, lmk_k = lmk_q.contiguous(), lmk_k.contiguous()
+    N, C, Dm = lmk_q.shape
+    E = lmk_k.shape[1]
+    assert lmk_k.shape[0] == N and lmk_k.shape[2] == Dm
+    hidden_size = Dm if hidden_size is None else hidden_size
+    scores = torch.empty((N, C, E), device=lmk_q.device, dtype=lmk_q.dtype)
+    desc = _lmk_desc(lmk_q.dtype, 1, N, C, E, Dm, causal, hidden_size)
+    with torch.cuda.device(lmk_q.device):
+        rc = _lib.lib().lmk_score(ctypes.byref(desc), _ptr(lmk_q), _ptr(lmk_k), _ptr(scores), _stream(lmk_q.device))
+    _lib.check(rc, "lmk_score")
+    return scores
+
+
+def landmark_topk(scores, topk, causal=True, noise=None):
+    """Top-k chunk ids and retrieval weights per row of ``scores`` (N, C, E)
+    (model/DRT.py:613-627).  Returns (indices int64 (N,C,kk), weights float32 (N,C,kk)) with
+    kk = min(E, topk); order: higher (score+noise) first, ties by lower index."""
+    assert scores.is_cuda and scores.dim() == 3 and scores.dtype in _DT
+    scores = scores.contiguous()
+    if noise is not None:
+        assert noise.shape == scores.shape and noise.dtype == scores.dtype
+        noise = noise.contiguous()
+    N, C, E = scores.shape
+    kk = min(E, int(topk))
+    indices = torch.empty((N, C, kk), device=scores.device, dtype=torch.int64)
+    weights = torch.empty((N, C, kk), device=scores.device, dtype=torch.float32)
+    desc = _lmk_desc(scores.dtype, topk, N, C, E, 1, causal, 1.0)
+    with torch.cuda.device(scores.device):
+        L = _lib.lib()
+        nbytes = L.lmk_topk_workspace_bytes(ctypes.byref(desc))
+        ws = torch.empty(max(nbytes // 8, 1), device=scores.device, dtype=torch.int64)
+        rc = L.lmk_topk(ctypes.byref(desc), _ptr(scores), _ptr(noise), _ptr(indices), _ptr(weights), _ptr(ws), nbytes,
+                        _stream(scores.device))
+    _lib.check(rc, "lmk_topk")
+    return indices, weights
+
+
+def landmark_retrieve(lmk_q, lmk_k, topk, hidden_size=None, causal=True, noise=None):
+    """Scoring + selection in one call.  Returns (scores, indices, weights)."""
+    scores = landmark_scores(lmk_q, lmk_k, hidden_size, causal)
+    indices, weights = landmark_topk(scores, topk, causal, noise)
+    return scores, indices, weights
+
+
+def gather_chunks(chunk_k, chunk_v, indices, weights, num_kv_heads):
+    """The reference's gather + layout (model/DRT.py:198-199, :629-637, :328-332): drops the
+    last retrieval row and returns k, v ((N (C-1)), Hkv, K, S, d) and weights ((N (C-1)), K).
+    Only needed by callers of the gathered-form ``attention``; ``attention_indexed`` reads the
+    cache directly."""
+    N, C, S, Dm = chunk_k.shape
+    K = indices.shape[-1]
+    d = Dm // num_kv_heads
+    idx = indices[:, :-1, :].reshape(N, (C - 1) * K)
+    bidx = torch.arange(N, device=chunk_k.device).unsqueeze(1)
+
+    def g(cache):
+        x = cache[bidx, idx].view(N, C - 1, K, S, num_kv_heads, d)
+        return x.permute(0, 1, 4, 2, 3, 5).reshape(N * (C - 1), num_kv_heads, K, S, d).contiguous()
+
+    return g(chunk_k), g(chunk_v), weights[:, :-1, :].reshape(N * (C - 1), K).contiguous()
+
+
+def gca_layer(q_all, chunk_k, chunk_v, lmk_q, lmk_k, topk, sm_n=0.0, hidden_size=None, noise=None, training=True):
+    """One GCA layer the way the reference wires it (model/DRT.py:345-398, :609-641), on the
+    indexed kernels: retrieval row c feeds query chunk c+1, chunk 0's output is zero,
+    sm_scale = 1/sqrt(d).  q_all (N, C, Hq, S, d); chunk_k/v (N, C, S, Hkv*d); lmk_q/k (N, C, Dm).
+    Returns (out (N, C, Hq, S, d), indices (N, C, kk), weights (N, C, kk))."""
+    from .gca import attention_indexed, gca_kv_cache_indexed
+    N, C, Hq, S, d = q_all.shape
+    _, indices, weights = landmark_retrieve(lmk_q, lmk_k, topk, hidden_size, True, noise)
+    out = torch.zeros_like(q_all)
+    if C > 1:
+        kk = indices.shape[-1]
+        q = q_all[:, 1:].reshape(N * (C - 1), Hq, S, d)
+        idx = indices[:, :-1].reshape(N * (C - 1), kk).contiguous()
+        w = weights[:, :-1].reshape(N * (C - 1), kk).contiguous()
+        fn = attention_indexed if training else gca_kv_cache_indexed
+        o = fn(q, chunk_k.contiguous(), chunk_v.contiguous(), idx, w, 1.0 / math.sqrt(d), sm_n)
+        out[:, 1:] = o.view(N, C - 1, Hq, S, d)
+    return out, indices, weights

@@ -1,0 +1,201 @@
+"""GPU parity of the GCA kernels against the CPU oracle, through the C ABI (ctypes).
+
+Tolerances (max |err| / max |ref|): 1e-5 for fp32, 2e-2 for bf16 -- the bars the task states;
+the reference's own test uses atol 1e-2 on o/dq/dk/dv and 0.5 on dw in bf16
+(ltriton/gca.py:938, :958-961), checked in test_reference_recipe."""
+import math
+
+import pytest
+import torch
+
+from helpers import gca_inputs, oracle64, rel_err, gen
+from oracle import gca_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
+
+
+def _run(q, k, v, w, do, sm_scale, sm_n, path="auto"):
+    import gca_hip
+    from gca_hip import gca as G
+    dev = torch.device("cuda:0")
+    qd, kd, vd, wd = [t.to(dev).requires_grad_(True) for t in (q, k, v, w)]
+    old = G.kernel_path
+    G.kernel_path = path
+    try:
+        o = gca_hip.attention(qd, kd, vd, wd, sm_scale, sm_n)
+        o.backward(do.to(dev))
+    finally:
+        G.kernel_path = old
+    torch.cuda.synchronize()
+    return o.detach(), qd.grad, kd.grad, vd.grad, wd.grad
+
+
+def _compare(got, ref, tol, names=("o", "dq", "dk", "dv", "dw")):
+    for n, a, b in zip(names, got, ref):
+        assert torch.isfinite(a.float()).all(), n
+        e = rel_err(a, b)
+        assert e <= tol, f"{n}: rel err {e:.3e} > {tol}"
+
+
+@pytest.mark.parametrize("sm_n", [0.0, 1.0])
+def test_cfg1_fp32(sm_n):
+    # BASELINE config 1: B=2, H=4, d=64, L=1024 (16 chunks of 64), top-k 4  ->  Z = 2*15
+    q, k, v, w, do = gca_inputs(30, 4, 4, 4, 64, 64, 64, torch.float32, seed=1)
+    ref = oracle64(q, k, v, w, do, 1 / 8, sm_n)
+    _compare(_run(q, k, v, w, do, 1 / 8, sm_n), ref, TOL[torch.float32])
+
+
+@pytest.mark.parametrize("path", ["generic", "auto"])
+@pytest.mark.parametrize("sm_n", [0.0, 1.0])
+def test_cfg2_shape_bf16_small_z(sm_n, path):
+    # BASELINE config 2 geometry (H=12, d=64, chunk 64, top-k 8) at a Z the oracle finishes in seconds
+    q, k, v, w, do = gca_inputs(6, 12, 12, 8, 64, 64, 64, torch.bfloat16, seed=2, w_dtype=torch.float32)
+    ref = oracle64(q, k, v, w, do, 1 / 8, sm_n)
+    _compare(_run(q, k, v, w, do, 1 / 8, sm_n, path), ref, TOL[torch.bfloat16])
+
+
+@pytest.mark.parametrize("path", ["generic", "auto"])
+def test_reference_recipe(path):
+    # ltriton/gca.py:891-961 at Z=8 instead of 512: H=40 (10 kv heads), K=32, d=64, N(0, 0.5), seed 22
+    torch.manual_seed(22)
+    Z, H, S, d, K = 8, 40, 64, 64, 32
+    dt = torch.bfloat16
+    q = torch.empty(Z, H, S, d, dtype=dt).normal_(0, 0.5)
+    k = torch.empty(Z, H // 4, K, S, d, dtype=dt).normal_(0, 0.5)
+    v = torch.empty(Z, H // 4, K, S, d, dtype=dt).normal_(0, 0.5)
+    w = torch.softmax(torch.rand(Z, K).to(dt), -1)
+    do = torch.randn(Z, H, S, d).to(dt)
+    ref = oracle64(q, k, v, w, do, 1 / 8, 0.0)
+    got = _run(q, k, v, w, do, 1 / 8, 0.0, path)
+    for n, a, b, atol in zip("o dq dk dv dw".split(), got, ref, (1e-2, 1e-2, 1e-2, 1e-2, 0.5)):
+        err = (a.double().cpu() - b).abs().max().item()
+        assert err <= atol, f"{n}: abs err {err:.3e} > {atol}"
+    _compare(got, ref, TOL[dt])
+
+
+@pytest.mark.parametrize("Q", [2, 1])
+def test_reference_decode_recipe(Q):
+    # ltriton/gca.py:963-1011: gca_kv_cache with Q_CTX 2 and 1, two query heads per kv head, sm_scale 0.5
+    import gca_hip
+    torch.manual_seed(22)
+    Z, H, S, d, K = 16, 40, 64, 64, 32
+    dt = torch.bfloat16
+    q = torch.empty(Z, H, Q, d, dtype=dt).normal_(0, 0.5)
+    k = torch.empty(Z, H // 2, K, S, d, dtype=dt).normal_(0, 0.5)
+    v = torch.empty(Z, H // 2, K, S, d, dtype=dt).normal_(0, 0.5)
+    w = torch.softmax(torch.rand(Z, K).to(dt), -1)
+    ref = orc.gca_forward(q.double(), k.double(), v.double(), w.double(), 0.5, 0.0)
+    got = gca_hip.gca_kv_cache(q.cuda(), k.cuda(), v.cuda(), w.cuda(), 0.5, 0.0)
+    assert got.shape == ref.shape and got.dtype == dt
+    assert (got.double().cpu() - ref).abs().max().item() <= 1e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [
+    # Z, Hq, Hkv, K, Q, S, d
+    (3, 4, 2, 3, 64, 64, 16),
+    (2, 4, 4, 5, 33, 80, 32),     # ragged query rows and key rows
+    (2, 8, 2, 16, 64, 64, 128),   # config-4 geometry: 4 query heads per kv head, d=128, top-k 16
+    (2, 2, 1, 2, 64, 48, 256),
+    (5, 6, 3, 1, 1, 64, 64),      # single query row, single retrieved chunk
+    (2, 2, 2, 4, 128, 64, 64),    # two 64-row tiles per chunk
+])
+def test_shapes_generic_and_auto(shape, dtype):
+    Z, Hq, Hkv, K, Q, S, d = shape
+    q, k, v, w, do = gca_inputs(Z, Hq, Hkv, K, Q, S, d, dtype, seed=3)
+    for sm_n in (0.0, 1.0):
+        ref = oracle64(q, k, v, w, do, 1 / math.sqrt(d), sm_n)
+        for path in ("generic", "auto"):
+            _compare(_run(q, k, v, w, do, 1 / math.sqrt(d), sm_n, path), ref, TOL[dtype])
+
+
+def test_masked_slots_and_zero_weights():
+    # slots whose weight is 0 (masked retrieval slots) contribute nothing and get zero dk/dv
+    q, k, v, w, do = gca_inputs(4, 4, 4, 4, 64, 64, 64, torch.bfloat16, seed=4, w_dtype=torch.float32)
+    w[:, 2:] = 0
+    w[0, :] = 0                       # a row with nothing retrieved at all
+    w = w / w.sum(-1, keepdim=True).clamp_min(1e-9)
+    ref = oracle64(q, k, v, w, do, 1 / 8, 1.0)
+    got = _run(q, k, v, w, do, 1 / 8, 1.0)
+    _compare(got, ref, TOL[torch.bfloat16])
+    assert got[0][0].abs().max() == 0
+    assert got[2][:, :, 2:].abs().max() == 0 and got[3][:, :, 2:].abs().max() == 0
+
+
+def test_zero_landmark_row_equals_softmax_one():
+    # zeroing one key/value row (model/DRT.py:772-779) == sm_n = 1 on the remaining 63 rows
+    import gca_hip
+    q, k, v, w, do = gca_inputs(3, 4, 4, 4, 64, 64, 64, torch.float32, seed=5)
+    k[:, :, :, -1] = 0
+    v[:, :, :, -1] = 0
+    a = gca_hip.gca_kv_cache(q.cuda(), k.cuda(), v.cuda(), w.cuda(), 1 / 8, 0.0)
+    b = gca_hip.gca_kv_cache(q.cuda(), k[:, :, :, :-1].contiguous().cuda(), v[:, :, :, :-1].contiguous().cuda(), w.cuda(), 1 / 8, 1.0)
+    assert rel_err(a, b) <= 1e-5
+
+
+def test_dropin_shim_matches_reference_kernel_arithmetic():
+    # the drop-in module ignores sm_n like the reference's kernels do (ltriton/gca.py:186-187, :48-49)
+    import ltriton.gca as shim
+    q, k, v, w, do = gca_inputs(3, 4, 4, 4, 64, 64, 64, torch.bfloat16, seed=6)
+    ref0 = orc.gca_forward(q.double(), k.double(), v.double(), w.double(), 1 / 8, 0.0)
+    ref1 = orc.gca_forward(q.double(), k.double(), v.double(), w.double(), 1 / 8, 1.0)
+    assert shim.SM_N_MODE == "reference"
+    got = shim.attention(q.cuda(), k.cuda(), v.cuda(), w.cuda(), 1 / 8, 1.0)
+    assert rel_err(got, ref0) <= TOL[torch.bfloat16]
+    shim.SM_N_MODE = "functional"
+    try:
+        got = shim.gca_kv_cache(q.cuda(), k.cuda(), v.cuda(), w.cuda(), 1 / 8, 1.0)
+        assert rel_err(got, ref1) <= TOL[torch.bfloat16]
+        assert rel_err(got, ref0) > 1e-3
+    finally:
+        shim.SM_N_MODE = "reference"
+
+
+def test_preconditions_raise_like_the_reference():
+    import gca_hip
+    q, k, v, w, do = [t.cuda() for t in gca_inputs(2, 4, 4, 2, 64, 64, 64, torch.bfloat16, seed=7)]
+    with pytest.raises(AssertionError):
+        gca_hip.attention(q.transpose(1, 2), k, v, w, 1 / 8, 0.0)                  # q not contiguous
+    with pytest.raises(AssertionError):
+        gca_hip.attention(q, k, v, w[:, :, None], 1 / 8, 0.0)                       # weights not 2-D
+    with pytest.raises(AssertionError):
+        gca_hip.attention(q[..., :48].contiguous(), k[..., :48].contiguous(), v[..., :48].contiguous(), w, 1 / 8, 0.0)
+    with pytest.raises(AssertionError):
+        gca_hip.attention(q[:, :3].contiguous(), k[:, :2].contiguous(), v[:, :2].contiguous(), w, 1 / 8, 0.0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_indexed_equals_gathered(dtype):
+    import gca_hip
+    N, C, S, Hq, Hkv, d, K = 2, 9, 64, 4, 2, 64, 4
+    ck = gen((N, C, S, Hkv * d), 10, 0.5, dtype)
+    cv = gen((N, C, S, Hkv * d), 11, 0.5, dtype)
+    g = torch.Generator().manual_seed(12)
+    idx = torch.randint(0, C, (N, C, K), generator=g)
+    idx[:, :, 1] = idx[:, :, 0]                                   # duplicates inside a row
+    idx[0, :, 2] = 3                                              # one chunk retrieved by every row
+    w = torch.softmax(torch.rand(N, C, K, generator=g), -1)
+    q = gen((N * (C - 1), Hq, S, d), 13, 0.5, dtype)
+    do = gen((N * (C - 1), Hq, S, d), 14, 1.0, dtype)
+    # oracle: gather, run, scatter-add the chunk gradients back into the cache (autograd does that)
+    ck64, cv64 = ck.double().requires_grad_(True), cv.double().requires_grad_(True)
+    q64, w64 = q.double().requires_grad_(True), w.double().requires_grad_(True)
+    kg, vg, wg = orc.gather_chunks(ck64, cv64, idx, w64, Hkv)
+    o_ref = orc.gca_forward(q64, kg, vg, wg, 1 / 8, 1.0)
+    o_ref.backward(do.double())
+    dev = "cuda"
+    qd, ckd, cvd = [t.to(dev).requires_grad_(True) for t in (q, ck, cv)]
+    wd = w[:, :-1].reshape(-1, K).contiguous().to(dev).requires_grad_(True)
+    idxd = idx[:, :-1].reshape(-1, K).contiguous().to(dev)
+    o = gca_hip.attention_indexed(qd, ckd, cvd, idxd, wd, 1 / 8, 1.0)
+    o.backward(do.to(dev))
+    tol = TOL[dtype]
+    assert rel_err(o, o_ref) <= tol
+    assert rel_err(qd.grad, q64.grad) <= tol
+    assert rel_err(ckd.grad, ck64.grad) <= tol
+    assert rel_err(cvd.grad, cv64.grad) <= tol
+    assert rel_err(wd.grad, w64.grad[:, :-1].reshape(-1, K)) <= tol
+    o2 = gca_hip.gca_kv_cache_indexed(qd.detach(), ckd.detach(), cvd.detach(), idxd, wd.detach(), 1 / 8, 1.0)
+    assert torch.equal(o2, o.detach())

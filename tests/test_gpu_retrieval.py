@@ -1,0 +1,143 @@
+"""GPU parity of landmark scoring / top-k / weights against the CPU oracle, through the C ABI.
+
+Index parity is exact: on given scores the kernel must return the oracle's indices slot by
+slot (including ties, -inf slots and rows with fewer than k visible chunks).  Where the
+kernel computes the scores itself they may differ from the CPU's in the last bit (different
+summation order), so there the selection is checked exactly against the canonical rule
+applied to the kernel's OWN scores, the scores against the oracle's within tolerance, and
+the indices against the oracle's wherever the oracle's gaps exceed that tolerance."""
+import math
+
+import pytest
+import torch
+
+from helpers import gen, rel_err
+from oracle import gca_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _topk_ref(scores, k, causal=True, noise=None):
+    """Oracle selection on given scores: mask, add the noise in the scores' own dtype for the
+    selection only, canonical top-k, weights from the noise-free masked scores."""
+    s = orc.mask_scores(scores.float()) if causal else scores.float()
+    sel = s
+    if noise is not None:
+        sel = (scores + noise).float()                      # rounded in the scores' dtype
+        sel = orc.mask_scores(sel) if causal else sel
+    kk = min(s.shape[-1], k)
+    _, idx = orc.topk_canonical(sel, kk)
+    return idx, orc.retrieval_weights(s, idx)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("N,C,k", [(2, 16, 4), (8, 256, 8), (1, 5, 8), (3, 70, 16), (1, 3000, 8), (1, 2100, 33)])
+def test_topk_exact_on_given_scores(N, C, k, dtype):
+    import gca_hip
+    scores = gen((N, C, C), 100 + C, 1.0, dtype)          # bf16 rows have many exact ties
+    idx_ref, w_ref = _topk_ref(scores, k)
+    idx, w = gca_hip.landmark_topk(scores.cuda(), k, causal=True)
+    assert idx.dtype == torch.int64 and idx.shape == idx_ref.shape
+    assert torch.equal(idx.cpu(), idx_ref)
+    assert (w.cpu() - w_ref).abs().max() <= 1e-6
+    assert (w.cpu()[orc.mask_scores(scores.float()).gather(2, idx_ref) == float('-inf')] == 0).all()
+    assert (w[:, 0] == 0).all()                            # row 0 sees nothing
+
+
+def test_topk_ties_and_special_values():
+    import gca_hip
+    g = torch.Generator().manual_seed(7)
+    scores = torch.randint(-2, 3, (2, 1, 500), generator=g).float()   # heavy ties, +-0 included
+    scores[0, 0, 17] = -0.0
+    scores[0, 0, 3] = float('inf')
+    scores[1, 0, 100:] = float('-inf')
+    idx_ref, w_ref = _topk_ref(scores, 16, causal=False)
+    idx, w = gca_hip.landmark_topk(scores.cuda(), 16, causal=False)
+    assert torch.equal(idx.cpu(), idx_ref)
+    assert torch.allclose(w.cpu(), w_ref, atol=1e-6, equal_nan=False)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_topk_gumbel_noise_selects_but_does_not_weigh(dtype):
+    import gca_hip
+    N, C, k = 2, 64, 8
+    scores = gen((N, C, C), 21, 1.0, dtype)
+    u = torch.rand(N, C, C, generator=torch.Generator().manual_seed(22)).clamp_min(1e-6)
+    noise = (-(-u.log()).log()).to(dtype)                  # Gumbel(0, 1), as model/DRT.py:617-620 draws it
+    idx_ref, w_ref = _topk_ref(scores, k, True, noise)
+    idx, w = gca_hip.landmark_topk(scores.cuda(), k, causal=True, noise=noise.cuda())
+    assert torch.equal(idx.cpu(), idx_ref)
+    assert (w.cpu() - w_ref).abs().max() <= 1e-6
+    assert not torch.equal(idx_ref, _topk_ref(scores, k)[0])
+
+
+def test_topk_long_row_uses_segments():
+    # one row long enough to be cut into segments and merged (decode at extreme context)
+    import gca_hip
+    E = 300_000
+    scores = gen((1, 1, E), 31, 1.0, torch.float32)
+    scores[0, 0, 123_456] = 9.0                             # needle
+    idx_ref, w_ref = _topk_ref(scores, 8)
+    idx, w = gca_hip.landmark_topk(scores.cuda(), 8, causal=True)
+    assert torch.equal(idx.cpu(), idx_ref) and idx[0, 0, 0] == 123_456
+    assert (w.cpu() - w_ref).abs().max() <= 1e-6
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("N,C,Dm,k", [(2, 16, 256, 4), (8, 256, 768, 8), (1, 37, 100, 5)])
+def test_score_topk(N, C, Dm, k, dtype, tol):
+    import gca_hip
+    lq, lk = gen((N, C, Dm), 41, 1.0, dtype), gen((N, C, Dm), 42, 1.0, dtype)
+    s_ref, idx_ref, w_ref = orc.retrieve(lq.double(), lk.double(), k, hidden_size=Dm)
+    scores, idx, w = gca_hip.landmark_retrieve(lq.cuda(), lk.cuda(), k, hidden_size=Dm)
+    sc = scores.float().cpu()
+    assert torch.equal(torch.isinf(sc), torch.isinf(s_ref))                  # same mask
+    fin = ~torch.isinf(s_ref)
+    err = (sc[fin].double() - s_ref[fin]).abs().max().item()
+    assert err <= tol * s_ref[fin].abs().max().item()
+    # exact w.r.t. the canonical rule on the kernel's own scores
+    idx_own, w_own = _topk_ref(scores.cpu(), k)
+    assert torch.equal(idx.cpu(), idx_own)
+    assert (w.cpu() - w_own).abs().max() <= 1e-6
+    # and equal to the oracle's indices wherever the oracle's choice is separated by more than the error
+    sel = s_ref.gather(2, idx_ref)
+    kk = idx_ref.shape[-1]
+    srt = torch.sort(s_ref, -1, descending=True).values[..., :kk + 1] if s_ref.shape[-1] > kk else None
+    gap_ok = torch.ones_like(idx_ref, dtype=torch.bool)
+    if srt is not None:
+        gaps = (srt[..., :-1] - srt[..., 1:])
+        gaps = torch.nan_to_num(gaps, nan=0.0, posinf=1e30)
+        safe = gaps > 4 * err
+        gap_ok = safe & torch.cat([torch.ones_like(safe[..., :1]), safe[..., :-1]], -1)
+    gap_ok &= ~torch.isinf(sel)
+    assert torch.equal(idx.cpu()[gap_ok], idx_ref[gap_ok])
+    assert gap_ok.float().mean() > (0.5 if dtype == torch.float32 else 0.05)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_decode_scan_scores(dtype):
+    # one query landmark against every cached landmark (model/DRT.py:836-844)
+    import gca_hip
+    N, E, Dm = 3, 1000, 768
+    lq, lk = gen((N, 1, Dm), 51, 1.0, dtype), gen((N, E, Dm), 52, 1.0, dtype)
+    s_ref = orc.mask_scores(orc.landmark_scores(lq.double(), lk.double(), Dm))
+    scores = gca_hip.landmark_scores(lq.cuda(), lk.cuda(), Dm, causal=True).float().cpu()
+    assert torch.isinf(scores[:, 0, -1]).all() and not torch.isinf(scores[:, 0, :-1]).any()
+    fin = ~torch.isinf(s_ref)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert (scores[fin].double() - s_ref[fin]).abs().max().item() <= tol * s_ref[fin].abs().max().item()
+
+
+def test_gca_layer_end_to_end_fp32():
+    # rows R1-R5 + the caller's row shift (model/DRT.py:345-398, :609-641), config-1 geometry
+    import gca_hip
+    N, C, H, S, d, K = 2, 16, 4, 64, 64, 4
+    q_all = gen((N, C, H, S, d), 61, 0.5)
+    ck, cv = gen((N, C, S, H * d), 62, 0.5), gen((N, C, S, H * d), 63, 0.5)
+    lq, lk = gen((N, C, H * d), 64), gen((N, C, H * d), 65)
+    out_ref, idx_ref, w_ref = orc.gca_layer(q_all.double(), ck.double(), cv.double(), lq.double(), lk.double(), K, H, sm_n=1.0)
+    out, idx, w = gca_hip.gca_layer(q_all.cuda(), ck.cuda(), cv.cuda(), lq.cuda(), lk.cuda(), K, sm_n=1.0, training=False)
+    assert torch.equal(idx.cpu(), idx_ref)
+    assert (w.cpu().double() - w_ref).abs().max() <= 1e-5
+    assert out[:, 0].abs().max() == 0
+    assert rel_err(out, out_ref) <= 1e-5
