@@ -1,7 +1,270 @@
-// placeholder until the MFMA forward lands
+// GCA forward on the gfx950 matrix cores (bf16 in, fp32 accumulate).
+//
+// Shape class: bf16, K_CTX == 64, D in {64, 128}, Q_CTX % 64 == 0, sm_scale > 0.
+//
+// Work split.  A workgroup owns one (z, kv head, slice of GS query heads of the group, 64-row
+// query tile) and walks the K retrieved chunks.  It has 2*GS wavefronts; wavefront w owns the
+// 32 query rows qb = w % 2 of query head w / 2.  Each retrieved chunk's K and V tiles
+// (64 x D bf16 each) are read from HBM once per workgroup with 16-byte coalesced loads,
+// staged in LDS (double buffered: the loads of chunk j+1 are issued before the math of chunk j),
+// and shared by all wavefronts.
+//
+// Per wavefront and chunk (v_mfma_f32_32x32x16_bf16, lane = (n = lane % 32, h = lane / 32)):
+//   S^T = K_j Q^T   A = K rows from LDS (16-byte reads), B = Q held in registers for the whole
+//                   kernel.  The result has keys in registers and the lane's own query n in every
+//                   register, so the softmax max/sum are in-lane reductions plus one exchange
+//                   with lane ^ 32.
+//   P~  = w_j exp2(c S - m) / l  rounded to bf16.  Its register layout already IS the A operand of
+//                   the second product (reduction index permuted the same way on both operands).
+//   O  += P~ V_j    B = V read from LDS with ds_read_tr16_b64, which hands each lane one dim
+//                   column of a 4-key x 16-dim patch, i.e. the transposed access V needs.
+// The softmax denominator includes sm_n * exp2(-m) (sm_n virtual keys of logit 0 and value 0).
+// lse[z, h, j, row] = m + log2(l) in the log2-scaled domain, written when lse != NULL.
 #include "gca_common.h"
+
 namespace gca {
-bool mfma_supported(const gca_desc&) { return false; }
-int launch_fwd_mfma(const gca_desc&, bool, const void*, const void*, const void*, const int64_t*, const void*, void*,
-                    float*, hipStream_t) { return GCA_ERR_UNSUPPORTED; }
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+
+template <int D> struct FwdCfg {
+    static constexpr int KSTRIDE = D * 2 + 16;   // bytes per K row in LDS: 16-byte reads of 8 rows hit distinct banks
+    static constexpr int VSTRIDE = D * 2 + 32;   // bytes per V row in LDS: 4-row transposed patches hit distinct banks
+    static constexpr int KBYTES = 64 * KSTRIDE;
+    static constexpr int VBYTES = 64 * VSTRIDE;
+    static constexpr int BUF = KBYTES + VBYTES;
+};
+
+__device__ __forceinline__ bf16x8 lds_read_b128(const unsigned char* p) {
+    return *reinterpret_cast<const bf16x8*>(p);
 }
+
+__device__ __forceinline__ bf16x8 lds_read_tr_pair(const unsigned char* p0, const unsigned char* p1) {
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p0);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p1);
+    union { s16x4 s[2]; bf16x8 v; } u;
+    u.s[0] = lo;
+    u.s[1] = hi;
+    return u.v;
+}
+
+template <int D, int GS, bool INDEXED>
+__global__ void __launch_bounds__(128 * GS)
+gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
+                    const uint16_t* __restrict__ v, const int64_t* __restrict__ indices,
+                    const void* __restrict__ w, int w_is_bf16, uint16_t* __restrict__ o, float* __restrict__ lse) {
+    using Cfg = FwdCfg<D>;
+    constexpr int NT = 128 * GS;
+    constexpr int KS = D / 16;                 // reduction steps of Q.K^T
+    constexpr int DB = D / 32;                 // 32-wide dim blocks of O
+    constexpr int PIECES = 64 * D * 2 / 16;    // 16-byte pieces per tile
+    constexpr int LPT = PIECES / NT;           // pieces per thread per tile
+    constexpr int PPR = D * 2 / 16;            // pieces per row
+    static_assert(PIECES % NT == 0, "tile must split evenly over the workgroup");
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * Cfg::BUF];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 31, h = lane >> 5;
+    const int gs = wave >> 1, qb = wave & 1;
+
+    // block -> (z, hk, slice, qt); consecutive blocks share z so that they touch neighbouring memory
+    const int nqt = p.Q_CTX / 64;
+    const int nslice = p.G / GS;
+    int64_t bid = blockIdx.x;
+    const int qt = (int)(bid % nqt); bid /= nqt;
+    const int slice = (int)(bid % nslice); bid /= nslice;
+    const int hk = (int)(bid % p.Hkv);
+    const int64_t z = bid / p.Hkv;
+    const int hq = hk * p.G + slice * GS + gs;
+    const int q0 = qt * 64 + qb * 32;
+
+    // Q as the B operand: lane holds row n, dims 16*ks + 8*h .. +7
+    bf16x8 qB[KS];
+    {
+        const uint16_t* qp = q + ((z * p.Hq + hq) * (int64_t)p.Q_CTX + q0 + n) * D + 8 * h;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qB[ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
+    }
+
+    f32x16 oacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
+
+    const float c = p.sm_scale * LOG2E;
+
+    // staging: thread owns pieces tid + i*NT of each tile; piece = (row, 16-byte column)
+    u32x4 stage_k[LPT], stage_v[LPT];
+    int64_t goff[LPT];      // element offset of the piece inside a chunk (row stride applied)
+    int lds_koff[LPT], lds_voff[LPT];
+    {
+        const int64_t rs = p.indexed ? (int64_t)p.Hkv * D : (int64_t)D;
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) {
+            const int piece = tid + i * NT;
+            const int row = piece / PPR, col = piece % PPR;
+            goff[i] = row * rs + col * 8;
+            lds_koff[i] = row * Cfg::KSTRIDE + col * 16;
+            lds_voff[i] = row * Cfg::VSTRIDE + col * 16;
+        }
+    }
+    {
+        int64_t rs;
+        const uint16_t* kj = chunk_base(p, k, indices, z, hk, 0, rs);
+        const uint16_t* vj = chunk_base(p, v, indices, z, hk, 0, rs);
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) {
+            stage_k[i] = *reinterpret_cast<const u32x4*>(kj + goff[i]);
+            stage_v[i] = *reinterpret_cast<const u32x4*>(vj + goff[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) {
+            *reinterpret_cast<u32x4*>(smem + lds_koff[i]) = stage_k[i];
+            *reinterpret_cast<u32x4*>(smem + Cfg::KBYTES + lds_voff[i]) = stage_v[i];
+        }
+    }
+    __syncthreads();
+
+    const int i16 = lane & 15;
+    const int dhalf = (lane >> 4) & 1;
+
+    for (int j = 0; j < p.K; ++j) {
+        const int buf = j & 1;
+        const bool more = (j + 1 < p.K);
+        if (more) {
+            int64_t rs;
+            const uint16_t* kj = chunk_base(p, k, indices, z, hk, j + 1, rs);
+            const uint16_t* vj = chunk_base(p, v, indices, z, hk, j + 1, rs);
+#pragma unroll
+            for (int i = 0; i < LPT; ++i) {
+                stage_k[i] = *reinterpret_cast<const u32x4*>(kj + goff[i]);
+                stage_v[i] = *reinterpret_cast<const u32x4*>(vj + goff[i]);
+            }
+        }
+
+        const unsigned char* kb = smem + buf * Cfg::BUF;
+        const unsigned char* vb = kb + Cfg::KBYTES;
+
+        // ---- S^T = K Q^T : two 32-key tiles, keys in registers, query n in the lane
+        f32x16 st[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) st[t][r] = 0.f;
+            const unsigned char* krow = kb + (32 * t + n) * Cfg::KSTRIDE + 16 * h;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const bf16x8 a = lds_read_b128(krow + 32 * ks);
+                st[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qB[ks], st[t], 0, 0, 0);
+            }
+        }
+
+        // ---- softmax over the 64 keys of this chunk for query n
+        float mx = st[0][0];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, st[t][r]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        float m2 = mx * c;
+        if (p.sm_n > 0.f) m2 = fmaxf(m2, 0.f);
+        float sum = 0.f;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float e = __builtin_amdgcn_exp2f(fmaf(st[t][r], c, -m2));
+                st[t][r] = e;
+                sum += e;
+            }
+        sum += __shfl_xor(sum, 32);
+        const float l = sum + p.sm_n * __builtin_amdgcn_exp2f(-m2);
+        const float wj = w_is_bf16 ? bf16_bits_to_f(((const uint16_t*)w)[z * p.K + j]) : ((const float*)w)[z * p.K + j];
+        const float inv = wj / l;
+        if (lse != nullptr && h == 0)
+            lse[((z * p.Hq + hq) * (int64_t)p.K + j) * p.Q_CTX + q0 + n] = m2 + __builtin_amdgcn_logf(l);
+
+        // ---- P~ as the A operand: step t4 covers keys 16*t4 .. +15; slots 0-3 = keys 16*t4 + 4h + c,
+        //      slots 4-7 = keys 16*t4 + 8 + 4h + c -- the S^T register order
+        bf16x8 pA[4];
+#pragma unroll
+        for (int t4 = 0; t4 < 4; ++t4)
+#pragma unroll
+            for (int s = 0; s < 8; ++s) pA[t4][s] = (__bf16)(st[t4 >> 1][8 * (t4 & 1) + s] * inv);
+
+        // ---- O += P~ V
+#pragma unroll
+        for (int t4 = 0; t4 < 4; ++t4) {
+            const unsigned char* vrow = vb + (16 * t4 + 4 * h + (i16 >> 2)) * Cfg::VSTRIDE + (16 * dhalf + 4 * (i16 & 3)) * 2;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const bf16x8 b = lds_read_tr_pair(vrow + 64 * db, vrow + 64 * db + 8 * Cfg::VSTRIDE);
+                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pA[t4], b, oacc[db], 0, 0, 0);
+            }
+        }
+
+        if (more) {
+            unsigned char* nb = smem + (buf ^ 1) * Cfg::BUF;
+#pragma unroll
+            for (int i = 0; i < LPT; ++i) {
+                *reinterpret_cast<u32x4*>(nb + lds_koff[i]) = stage_k[i];
+                *reinterpret_cast<u32x4*>(nb + Cfg::KBYTES + lds_voff[i]) = stage_v[i];
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- store O: register r of block db is row 8*(r/4) + 4*h + r%4, column 32*db + n
+    uint16_t* op = o + ((z * p.Hq + hq) * (int64_t)p.Q_CTX + q0) * D;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = 8 * (r >> 2) + 4 * h + (r & 3);
+            const __bf16 ob = (__bf16)oacc[db][r];
+            op[row * D + 32 * db + n] = __builtin_bit_cast(uint16_t, ob);
+        }
+}
+
+bool mfma_supported(const gca_desc& d) {
+    return d.dtype == GCA_BF16 && d.K_CTX == 64 && (d.D == 64 || d.D == 128) && d.Q_CTX % 64 == 0 && d.sm_scale > 0.f;
+}
+
+template <int D, int GS>
+static int launch_gs(const Params& p, const void* q, const void* k, const void* v, const int64_t* idx,
+                     const void* w, int w_is_bf16, void* o, float* lse, hipStream_t s) {
+    const int64_t blocks = p.Z * p.Hkv * (p.G / GS) * (p.Q_CTX / 64);
+    if (blocks <= 0 || blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
+    if (p.indexed)
+        hipLaunchKernelGGL((gca_fwd_mfma_kernel<D, GS, true>), dim3((unsigned)blocks), dim3(128 * GS), 0, s, p,
+                           (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, idx, w, w_is_bf16, (uint16_t*)o, lse);
+    else
+        hipLaunchKernelGGL((gca_fwd_mfma_kernel<D, GS, false>), dim3((unsigned)blocks), dim3(128 * GS), 0, s, p,
+                           (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, idx, w, w_is_bf16, (uint16_t*)o, lse);
+    return hipGetLastError() == hipSuccess ? GCA_OK : GCA_ERR_LAUNCH;
+}
+
+template <int D>
+static int launch_d(const Params& p, const void* q, const void* k, const void* v, const int64_t* idx,
+                    const void* w, int w_is_bf16, void* o, float* lse, hipStream_t s) {
+    if (p.G % 4 == 0) return launch_gs<D, 4>(p, q, k, v, idx, w, w_is_bf16, o, lse, s);
+    if (p.G % 2 == 0) return launch_gs<D, 2>(p, q, k, v, idx, w, w_is_bf16, o, lse, s);
+    return launch_gs<D, 1>(p, q, k, v, idx, w, w_is_bf16, o, lse, s);
+}
+
+int launch_fwd_mfma(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v,
+                    const int64_t* indices, const void* w, void* o, float* lse, hipStream_t s) {
+    if (!mfma_supported(d)) return GCA_ERR_UNSUPPORTED;
+    const Params p = make_params(d, indexed);
+    const int wb = d.w_dtype == GCA_BF16 ? 1 : 0;
+    if (d.D == 64) return launch_d<64>(p, q, k, v, indices, w, wb, o, lse, s);
+    return launch_d<128>(p, q, k, v, indices, w, wb, o, lse, s);
+}
+
+}  // namespace gca
