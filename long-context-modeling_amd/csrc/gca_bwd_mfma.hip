@@ -1,9 +1,588 @@
-// placeholder until the MFMA backward lands: the generic backward consumes the same lse
-#include "gca_common.h"
+// GCA backward on the gfx950 matrix cores (bf16 in, fp32 accumulate).  Same shape class as the
+// MFMA forward: bf16, K_CTX == 64, D in {64, 128}, Q_CTX % 64 == 0, sm_scale > 0.
+//
+// Two kernels, five + two products per (query head, retrieved chunk):
+//
+// 1. dq kernel -- query-centric, the forward's work split (workgroup = (z, kv head, GS query heads,
+//    64 query rows), wavefront = 32 query rows, K/V tiles of the retrieved chunks double-buffered in LDS).
+//      S^T = K Q^T, dP^T = V dO^T        keys in registers, the lane's query in every register
+//      P = exp2(c S - lse), D = rowsum(P * dP)  (in-lane sums + one exchange), stored to `delta`
+//      dS = w sm_scale P (dP - D) -> bf16, already in A-operand order
+//      dQ += dS K                         K read transposed from LDS (ds_read_tr16_b64)
+//
+// 2. dkdv kernel -- kv-tile-centric.  A workgroup owns ONE 64 x D key/value tile (its two wavefronts
+//    own 32 key rows each, K and V rows held in registers as B operands) and walks every
+//    (query chunk z, slot j, query head of the group, 64-row query tile) that attends to this tile; Q and dO tiles are
+//    staged in LDS (double buffered) and shared by both wavefronts.
+//      S = Q K^T, dP = dO V^T            queries in registers, the lane's key in every register
+//      P = exp2(c S - lse[q]), P~ = w P, dS = sm_scale P~ (dP - delta[q])   lse/delta rows from LDS
+//      dV += P~^T dO,  dK += dS^T Q      dO and Q read transposed from LDS
+//    Gathered form: the tile is slot (z, kv head, j) and the walk is the G heads of the group; dk/dv
+//    are written in bf16.  Indexed form: the tile is a chunk of the cache and the walk follows a
+//    reference list built on the device (count -> scan -> fill, every list ordered by (z, j), no
+//    atomics, so the summation order is fixed).  Lists longer than SEG_MAX are cut into segments handled by
+//    separate workgroups; only those chunks use float atomics, all others store directly.
+//
+// dw[z, j] = sum over heads and rows of delta (shared launch_dw).
+#include "gca_mfma.h"
+
 namespace gca {
+
+int launch_dw(const Params& p, const float* delta, float* dw, hipStream_t s);
+
+constexpr int SEG_MAX = 16;   // references per dkdv workgroup in the indexed form
+
+// ------------------------------------------------------------------------------------------- dq
+
+template <int D, int GS, bool INDEXED>
+__global__ void __launch_bounds__(128 * GS)
+gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
+                       const uint16_t* __restrict__ v, const int64_t* __restrict__ indices,
+                       const void* __restrict__ w, int w_is_bf16, const uint16_t* __restrict__ dout,
+                       const float* __restrict__ lse, uint16_t* __restrict__ dq, float* __restrict__ delta) {
+    constexpr int NT = 128 * GS;
+    constexpr int KS = D / 16, DB = D / 32;
+    constexpr int RB = D * 2, TILE = 64 * RB, BUF = 2 * TILE;
+    constexpr int PIECES = TILE / 16, LPT = PIECES / NT, PPR = RB / 16;
+    static_assert(PIECES % NT == 0, "tile must split evenly over the workgroup");
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 31, h = lane >> 5;
+    const int gs = wave >> 1, qb = wave & 1;
+    const int nqt = p.Q_CTX / 64, nslice = p.G / GS;
+    int64_t bid = blockIdx.x;
+    const int qt = (int)(bid % nqt); bid /= nqt;
+    const int slice = (int)(bid % nslice); bid /= nslice;
+    const int hk = (int)(bid % p.Hkv);
+    const int64_t z = bid / p.Hkv;
+    const int hq = hk * p.G + slice * GS + gs;
+    const int q0 = qt * 64 + qb * 32;
+
+    bf16x8 qB[KS], doB[KS];
+    {
+        const int64_t off = ((z * p.Hq + hq) * (int64_t)p.Q_CTX + q0 + n) * D + 8 * h;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            qB[ks] = *reinterpret_cast<const bf16x8*>(q + off + 16 * ks);
+            doB[ks] = *reinterpret_cast<const bf16x8*>(dout + off + 16 * ks);
+        }
+    }
+    f32x16 dqacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dqacc[db][r] = 0.f;
+
+    const float c = p.sm_scale * LOG2E;
+    u32x4 stage_k[LPT], stage_v[LPT];
+    int64_t goff[LPT];
+    int loff[LPT];
+    {
+        const int64_t rs = INDEXED ? (int64_t)p.Hkv * D : (int64_t)D;
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) {
+            const int piece = tid + i * NT;
+            const int row = piece / PPR, col = piece % PPR;
+            goff[i] = row * rs + col * 8;
+            loff[i] = tile_off(row, col, RB);
+        }
+    }
+    {
+        int64_t rs;
+        const uint16_t* kj = chunk_base(p, k, indices, z, hk, 0, rs);
+        const uint16_t* vj = chunk_base(p, v, indices, z, hk, 0, rs);
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) {
+            stage_k[i] = *reinterpret_cast<const u32x4*>(kj + goff[i]);
+            stage_v[i] = *reinterpret_cast<const u32x4*>(vj + goff[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) {
+            *reinterpret_cast<u32x4*>(smem + loff[i]) = stage_k[i];
+            *reinterpret_cast<u32x4*>(smem + TILE + loff[i]) = stage_v[i];
+        }
+    }
+    __syncthreads();
+
+    const TrLane tr(lane);
+    const int fsw = swz(n);
+    const int64_t lrow = (z * p.Hq + hq) * (int64_t)p.K * p.Q_CTX + q0 + n;
+
+    for (int j = 0; j < p.K; ++j) {
+        const int buf = j & 1;
+        const bool more = (j + 1 < p.K);
+        if (more) {
+            int64_t rs;
+            const uint16_t* kj = chunk_base(p, k, indices, z, hk, j + 1, rs);
+            const uint16_t* vj = chunk_base(p, v, indices, z, hk, j + 1, rs);
+#pragma unroll
+            for (int i = 0; i < LPT; ++i) {
+                stage_k[i] = *reinterpret_cast<const u32x4*>(kj + goff[i]);
+                stage_v[i] = *reinterpret_cast<const u32x4*>(vj + goff[i]);
+            }
+        }
+        const float lse_q = lse[lrow + (int64_t)j * p.Q_CTX];
+        const float mult = load_w(w, w_is_bf16, z * p.K + j) * p.sm_scale;
+        const unsigned char* kb = smem + buf * BUF;
+        const unsigned char* vb = kb + TILE;
+
+        f32x16 st[2], dpt[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { st[t][r] = 0.f; dpt[t][r] = 0.f; }
+            const int rowoff = (32 * t + n) * RB;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int po = rowoff + (((2 * ks + h) ^ fsw) << 4);
+                st[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(kb + po), qB[ks], st[t], 0, 0, 0);
+                dpt[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(vb + po), doB[ks], dpt[t], 0, 0, 0);
+            }
+        }
+        float dsum = 0.f;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float pe = __builtin_amdgcn_exp2f(fmaf(st[t][r], c, -lse_q));
+                st[t][r] = pe;
+                dsum = fmaf(pe, dpt[t][r], dsum);
+            }
+        dsum += __shfl_xor(dsum, 32);
+        if (h == 0) delta[lrow + (int64_t)j * p.Q_CTX] = dsum;
+
+        bf16x8 dsA[4];
+#pragma unroll
+        for (int t4 = 0; t4 < 4; ++t4)
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                const int r = 8 * (t4 & 1) + s;
+                dsA[t4][s] = (__bf16)(st[t4 >> 1][r] * (dpt[t4 >> 1][r] - dsum) * mult);
+            }
+#pragma unroll
+        for (int t4 = 0; t4 < 4; ++t4)
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const int o0 = tr.off(t4, db, RB);
+                const bf16x8 b = lds_read_tr_pair(kb + o0, kb + o0 + 8 * RB);
+                dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsA[t4], b, dqacc[db], 0, 0, 0);
+            }
+
+        if (more) {
+            unsigned char* nb = smem + (buf ^ 1) * BUF;
+#pragma unroll
+            for (int i = 0; i < LPT; ++i) {
+                *reinterpret_cast<u32x4*>(nb + loff[i]) = stage_k[i];
+                *reinterpret_cast<u32x4*>(nb + TILE + loff[i]) = stage_v[i];
+            }
+        }
+        __syncthreads();
+    }
+
+    uint16_t* dqp = dq + ((z * p.Hq + hq) * (int64_t)p.Q_CTX + q0) * D;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = 8 * (r >> 2) + 4 * h + (r & 3);
+            dqp[row * D + 32 * db + n] = bf16_bits(dqacc[db][r]);
+        }
+}
+
+// ------------------------------------------------------------------------------------------- lists
+
+// Reference lists of the indexed form.  Chunk cc = n*C + c of the cache is referenced by
+// ref = z*K + j whenever indices[z, j] == c and z belongs to sequence n.
+struct ListWs {
+    int* count;      // [NC]      references per chunk
+    int* start;      // [NC]      first slot of the chunk's list in refs
+    int* seg_base;   // [NC]      first segment of the chunk
+    int* nseg;       // [1]       total segments
+    int* refs;       // [Z*K]     reference ids, chunk by chunk, each list ascending
+    int* seg_chunk;  // [bound]   chunk of a segment
+    int* seg_start;  // [bound]   first slot in refs
+    int* seg_len;    // [bound]   references in the segment (<= SEG_MAX)
+    int* seg_multi;  // [bound]   1 if the chunk has more than one segment
+};
+
+static inline int64_t seg_bound(const Params& p) { return p.N * p.C + (p.Z * p.K + SEG_MAX - 1) / SEG_MAX; }
+
+static inline size_t list_ws_ints(const Params& p) {
+    return (size_t)(3 * p.N * p.C + 4 + p.Z * p.K + 4 * seg_bound(p));
+}
+
+static ListWs carve_list_ws(const Params& p, int* base) {
+    ListWs ws;
+    const int64_t NC = p.N * p.C, sb = seg_bound(p);
+    ws.count = base; base += NC;
+    ws.start = base; base += NC;
+    ws.seg_base = base; base += NC;
+    ws.nseg = base; base += 4;
+    ws.refs = base; base += p.Z * p.K;
+    ws.seg_chunk = base; base += sb;
+    ws.seg_start = base; base += sb;
+    ws.seg_len = base; base += sb;
+    ws.seg_multi = base;
+    return ws;
+}
+
+__device__ __forceinline__ int64_t clamp_idx(int64_t c, int64_t C) { return c < 0 ? 0 : (c >= C ? C - 1 : c); }
+
+__global__ void __launch_bounds__(256)
+gca_bwd_list_count_kernel(Params p, const int64_t* __restrict__ indices, ListWs ws) {
+    const int64_t cc = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (cc >= p.N * p.C) return;
+    const int64_t n = cc / p.C, c = cc % p.C;
+    const int64_t r0 = n * p.zpn * p.K, r1 = r0 + p.zpn * p.K;
+    int cnt = 0;
+    for (int64_t r = r0; r < r1; ++r) cnt += (clamp_idx(indices[r], p.C) == c) ? 1 : 0;
+    ws.count[cc] = cnt;
+}
+
+// one workgroup: exclusive scans of the counts (list starts) and of the segment counts
+__global__ void __launch_bounds__(1024)
+gca_bwd_list_scan_kernel(Params p, ListWs ws) {
+    __shared__ int s_cnt[1024], s_seg[1024];
+    __shared__ int carry_cnt, carry_seg;
+    const int tid = threadIdx.x;
+    const int64_t NC = p.N * p.C;
+    if (tid == 0) { carry_cnt = 0; carry_seg = 0; }
+    __syncthreads();
+    for (int64_t base = 0; base < NC; base += 1024) {
+        const int64_t cc = base + tid;
+        const int cnt = cc < NC ? ws.count[cc] : 0;
+        const int sg = (cnt + SEG_MAX - 1) / SEG_MAX;
+        s_cnt[tid] = cnt;
+        s_seg[tid] = sg;
+        __syncthreads();
+        for (int off = 1; off < 1024; off <<= 1) {
+            const int a = tid >= off ? s_cnt[tid - off] : 0;
+            const int b = tid >= off ? s_seg[tid - off] : 0;
+            __syncthreads();
+            s_cnt[tid] += a;
+            s_seg[tid] += b;
+            __syncthreads();
+        }
+        if (cc < NC) {
+            ws.start[cc] = carry_cnt + s_cnt[tid] - cnt;
+            ws.seg_base[cc] = carry_seg + s_seg[tid] - sg;
+        }
+        __syncthreads();
+        if (tid == 1023) { carry_cnt += s_cnt[1023]; carry_seg += s_seg[1023]; }
+        __syncthreads();
+    }
+    if (tid == 0) ws.nseg[0] = carry_seg;
+}
+
+__global__ void __launch_bounds__(256)
+gca_bwd_list_fill_kernel(Params p, const int64_t* __restrict__ indices, ListWs ws) {
+    const int64_t cc = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (cc >= p.N * p.C) return;
+    const int64_t n = cc / p.C, c = cc % p.C;
+    const int64_t r0 = n * p.zpn * p.K, r1 = r0 + p.zpn * p.K;
+    const int start = ws.start[cc], cnt = ws.count[cc];
+    int kfill = 0;
+    for (int64_t r = r0; r < r1 && kfill < cnt; ++r)
+        if (clamp_idx(indices[r], p.C) == c) ws.refs[start + kfill++] = (int)r;
+    const int sg = (cnt + SEG_MAX - 1) / SEG_MAX, sb = ws.seg_base[cc];
+    for (int s = 0; s < sg; ++s) {
+        ws.seg_chunk[sb + s] = (int)cc;
+        ws.seg_start[sb + s] = start + s * SEG_MAX;
+        ws.seg_len[sb + s] = min(SEG_MAX, cnt - s * SEG_MAX);
+        ws.seg_multi[sb + s] = sg > 1 ? 1 : 0;
+    }
+}
+
+// ------------------------------------------------------------------------------------------- dkdv
+
+template <int D, bool INDEXED>
+__global__ void __launch_bounds__(128)
+gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
+                         const uint16_t* __restrict__ v, const void* __restrict__ w, int w_is_bf16,
+                         const uint16_t* __restrict__ dout, const float* __restrict__ lse,
+                         const float* __restrict__ delta, void* __restrict__ dk_out, void* __restrict__ dv_out,
+                         ListWs ws) {
+    constexpr int NT = 128;
+    constexpr int KS = D / 16, DB = D / 32;
+    constexpr int RB = D * 2, TILE = 64 * RB, BUF = 2 * TILE;   // Q tile then dO tile
+    constexpr int PIECES = TILE / 16, LPT = PIECES / NT, PPR = RB / 16;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF];
+    __shared__ __attribute__((aligned(16))) float s_lse[2][64];
+    __shared__ __attribute__((aligned(16))) float s_dl[2][64];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, kbw = tid >> 6;     // kbw: which 32 key rows this wavefront owns
+    const int n = lane & 31, h = lane >> 5;
+
+    // ---- which tile, which walk
+    int hk, nunits, list0 = 0, multi = 0;
+    int64_t gz = 0;          // gathered: the single (z, j)
+    int gj = 0;
+    const uint16_t* kt;
+    const uint16_t* vt;
+    int64_t rs, out_off;     // key-row stride of the tile; element offset of the tile in the output
+    if (INDEXED) {
+        const int seg = blockIdx.x / p.Hkv;
+        hk = blockIdx.x % p.Hkv;
+        if (seg >= ws.nseg[0]) return;
+        const int64_t cc = ws.seg_chunk[seg];
+        list0 = ws.seg_start[seg];
+        nunits = ws.seg_len[seg] * p.G * (p.Q_CTX / 64);
+        multi = ws.seg_multi[seg];
+        rs = (int64_t)p.Hkv * D;
+        out_off = cc * p.K_CTX * rs + (int64_t)hk * D;
+        kt = k + out_off;
+        vt = v + out_off;
+    } else {
+        int64_t bid = blockIdx.x;
+        gj = (int)(bid % p.K); bid /= p.K;
+        hk = (int)(bid % p.Hkv);
+        gz = bid / p.Hkv;
+        nunits = p.G * (p.Q_CTX / 64);
+        rs = D;
+        out_off = (((gz * p.Hkv + hk) * p.K + gj) * (int64_t)p.K_CTX) * D;
+        kt = k + out_off;
+        vt = v + out_off;
+    }
+
+    // K, V rows of this wavefront as B operands: lane holds key 32*kbw + n, dims 16*ks + 8*h .. +7
+    bf16x8 kB[KS], vB[KS];
+    {
+        const int64_t off = (int64_t)(32 * kbw + n) * rs + 8 * h;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            kB[ks] = *reinterpret_cast<const bf16x8*>(kt + off + 16 * ks);
+            vB[ks] = *reinterpret_cast<const bf16x8*>(vt + off + 16 * ks);
+        }
+    }
+    f32x16 dkacc[DB], dvacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
+
+    const float c = p.sm_scale * LOG2E;
+    u32x4 stage_q[LPT], stage_do[LPT];
+    float stage_f = 0.f;    // threads 0-63 stage lse[q], threads 64-127 stage delta[q]
+    int goff[LPT], loff[LPT];
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+        const int piece = tid + i * NT;
+        const int row = piece / PPR, col = piece % PPR;
+        goff[i] = row * D + col * 8;
+        loff[i] = tile_off(row, col, RB);
+    }
+
+    // unit u = (reference, query head of the group, 64-row query tile), tile fastest
+    const int nqt = p.Q_CTX / 64;
+    const int upr = p.G * nqt;   // units per reference
+    auto unit_coords = [&](int u, int64_t& z, int& j, int& hq, int& qrow0) {
+        const int g = (u % upr) / nqt;
+        qrow0 = (u % nqt) * 64;
+        hq = hk * p.G + g;
+        if (INDEXED) {
+            const int ref = ws.refs[list0 + u / upr];
+            z = ref / p.K;
+            j = ref % p.K;
+        } else {
+            z = gz;
+            j = gj;
+        }
+    };
+
+    float w_cur, w_next = 0.f;
+    {
+        int64_t z; int j, hq, qrow0;
+        unit_coords(0, z, j, hq, qrow0);
+        const int64_t qoff = ((z * p.Hq + hq) * (int64_t)p.Q_CTX + qrow0) * D;
+        const int64_t loffq = ((z * p.Hq + hq) * (int64_t)p.K + j) * p.Q_CTX + qrow0;
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) {
+            stage_q[i] = *reinterpret_cast<const u32x4*>(q + qoff + goff[i]);
+            stage_do[i] = *reinterpret_cast<const u32x4*>(dout + qoff + goff[i]);
+        }
+        stage_f = tid < 64 ? lse[loffq + tid] : delta[loffq + tid - 64];
+        w_cur = load_w(w, w_is_bf16, z * p.K + j);
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) {
+            *reinterpret_cast<u32x4*>(smem + loff[i]) = stage_q[i];
+            *reinterpret_cast<u32x4*>(smem + TILE + loff[i]) = stage_do[i];
+        }
+        if (tid < 64) s_lse[0][tid] = stage_f; else s_dl[0][tid - 64] = stage_f;
+    }
+    __syncthreads();
+
+    const TrLane tr(lane);
+    const int fsw = swz(n);
+
+    for (int u = 0; u < nunits; ++u) {
+        const int buf = u & 1;
+        const bool more = (u + 1 < nunits);
+        if (more) {
+            int64_t z; int j, hq, qrow0;
+            unit_coords(u + 1, z, j, hq, qrow0);
+            const int64_t qoff = ((z * p.Hq + hq) * (int64_t)p.Q_CTX + qrow0) * D;
+            const int64_t loffq = ((z * p.Hq + hq) * (int64_t)p.K + j) * p.Q_CTX + qrow0;
+#pragma unroll
+            for (int i = 0; i < LPT; ++i) {
+                stage_q[i] = *reinterpret_cast<const u32x4*>(q + qoff + goff[i]);
+                stage_do[i] = *reinterpret_cast<const u32x4*>(dout + qoff + goff[i]);
+            }
+            stage_f = tid < 64 ? lse[loffq + tid] : delta[loffq + tid - 64];
+            w_next = load_w(w, w_is_bf16, z * p.K + j);
+        }
+        const unsigned char* qbuf = smem + buf * BUF;
+        const unsigned char* dobuf = qbuf + TILE;
+        const float wj = w_cur, wsj = w_cur * p.sm_scale;
+
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) {
+            // S = Q K^T, dP = dO V^T for 32 query rows: queries in registers, key n in the lane
+            f32x16 s, dp;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+            const int rowoff = (32 * qt + n) * RB;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int po = rowoff + (((2 * ks + h) ^ fsw) << 4);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(qbuf + po), kB[ks], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(dobuf + po), vB[ks], dp, 0, 0, 0);
+            }
+            bf16x8 pA[2], dsA[2];
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                // registers 4a .. 4a+3 are queries 32*qt + 8a + 4h + 0..3
+                const f32x4 l4 = *reinterpret_cast<const f32x4*>(&s_lse[buf][32 * qt + 8 * a + 4 * h]);
+                const f32x4 d4 = *reinterpret_cast<const f32x4*>(&s_dl[buf][32 * qt + 8 * a + 4 * h]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int r = 4 * a + e;
+                    const float pe = __builtin_amdgcn_exp2f(fmaf(s[r], c, -l4[e]));
+                    pA[r >> 3][r & 7] = (__bf16)(pe * wj);
+                    dsA[r >> 3][r & 7] = (__bf16)(pe * (dp[r] - d4[e]) * wsj);
+                }
+            }
+            // dV += P~^T dO, dK += dS^T Q over these 32 queries (two 16-query reduction steps)
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+                const int t4 = 2 * qt + t2;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    const int o0 = tr.off(t4, db, RB);
+                    const bf16x8 bdo = lds_read_tr_pair(dobuf + o0, dobuf + o0 + 8 * RB);
+                    dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pA[t2], bdo, dvacc[db], 0, 0, 0);
+                    const bf16x8 bq = lds_read_tr_pair(qbuf + o0, qbuf + o0 + 8 * RB);
+                    dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsA[t2], bq, dkacc[db], 0, 0, 0);
+                }
+            }
+        }
+
+        if (more) {
+            unsigned char* nb = smem + (buf ^ 1) * BUF;
+#pragma unroll
+            for (int i = 0; i < LPT; ++i) {
+                *reinterpret_cast<u32x4*>(nb + loff[i]) = stage_q[i];
+                *reinterpret_cast<u32x4*>(nb + TILE + loff[i]) = stage_do[i];
+            }
+            if (tid < 64) s_lse[buf ^ 1][tid] = stage_f; else s_dl[buf ^ 1][tid - 64] = stage_f;
+            w_cur = w_next;
+        }
+        __syncthreads();
+    }
+
+    // ---- write the tile: register r of block db is key row 32*kbw + 8*(r/4) + 4*h + r%4, column 32*db + n
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = 32 * kbw + 8 * (r >> 2) + 4 * h + (r & 3);
+            const int64_t off = out_off + (int64_t)row * rs + 32 * db + n;
+            if (INDEXED) {
+                if (multi) {
+                    atomicAdd((float*)dk_out + off, dkacc[db][r]);
+                    atomicAdd((float*)dv_out + off, dvacc[db][r]);
+                } else {
+                    ((float*)dk_out)[off] = dkacc[db][r];
+                    ((float*)dv_out)[off] = dvacc[db][r];
+                }
+            } else {
+                ((uint16_t*)dk_out)[off] = bf16_bits(dkacc[db][r]);
+                ((uint16_t*)dv_out)[off] = bf16_bits(dvacc[db][r]);
+            }
+        }
+}
+
+// ------------------------------------------------------------------------------------------- launch
+
+template <int D, int GS>
+static int launch_dq_gs(const Params& p, const void* q, const void* k, const void* v, const int64_t* idx, const void* w,
+                        int wb, const void* dout, const float* lse, void* dq, float* delta, hipStream_t s) {
+    const int64_t blocks = p.Z * p.Hkv * (p.G / GS) * (p.Q_CTX / 64);
+    if (blocks <= 0 || blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
+    if (p.indexed)
+        hipLaunchKernelGGL((gca_bwd_dq_mfma_kernel<D, GS, true>), dim3((unsigned)blocks), dim3(128 * GS), 0, s, p,
+                           (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, idx, w, wb, (const uint16_t*)dout, lse,
+                           (uint16_t*)dq, delta);
+    else
+        hipLaunchKernelGGL((gca_bwd_dq_mfma_kernel<D, GS, false>), dim3((unsigned)blocks), dim3(128 * GS), 0, s, p,
+                           (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, idx, w, wb, (const uint16_t*)dout, lse,
+                           (uint16_t*)dq, delta);
+    return hipGetLastError() == hipSuccess ? GCA_OK : GCA_ERR_LAUNCH;
+}
+
+template <int D>
+static int launch_bwd_d(const Params& p, const void* q, const void* k, const void* v, const int64_t* idx, const void* w,
+                        int wb, const void* dout, const float* lse, void* dq, void* dk, void* dv, float* dw,
+                        float* delta, hipStream_t s) {
+    int rc;
+    if (p.G % 4 == 0) rc = launch_dq_gs<D, 4>(p, q, k, v, idx, w, wb, dout, lse, dq, delta, s);
+    else if (p.G % 2 == 0) rc = launch_dq_gs<D, 2>(p, q, k, v, idx, w, wb, dout, lse, dq, delta, s);
+    else rc = launch_dq_gs<D, 1>(p, q, k, v, idx, w, wb, dout, lse, dq, delta, s);
+    if (rc != GCA_OK) return rc;
+
+    ListWs ws = {};
+    if (p.indexed) {
+        // the list workspace follows delta
+        int* base = (int*)(delta + (size_t)p.Z * p.Hq * p.K * p.Q_CTX);
+        ws = carve_list_ws(p, base);
+        const int64_t NC = p.N * p.C;
+        const unsigned nb = (unsigned)((NC + 255) / 256);
+        hipLaunchKernelGGL(gca_bwd_list_count_kernel, dim3(nb), dim3(256), 0, s, p, idx, ws);
+        hipLaunchKernelGGL(gca_bwd_list_scan_kernel, dim3(1), dim3(1024), 0, s, p, ws);
+        hipLaunchKernelGGL(gca_bwd_list_fill_kernel, dim3(nb), dim3(256), 0, s, p, idx, ws);
+        if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
+        const int64_t blocks = seg_bound(p) * p.Hkv;
+        if (blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
+        hipLaunchKernelGGL((gca_bwd_dkdv_mfma_kernel<D, true>), dim3((unsigned)blocks), dim3(128), 0, s, p,
+                           (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse, delta,
+                           dk, dv, ws);
+    } else {
+        const int64_t blocks = p.Z * p.Hkv * p.K;
+        if (blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
+        hipLaunchKernelGGL((gca_bwd_dkdv_mfma_kernel<D, false>), dim3((unsigned)blocks), dim3(128), 0, s, p,
+                           (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse, delta,
+                           dk, dv, ws);
+    }
+    if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
+    return launch_dw(p, delta, dw, s);
+}
+
+size_t bwd_workspace_bytes(const gca_desc& d, bool indexed) {
+    size_t bytes = (size_t)d.Z * d.Hq * d.K * d.Q_CTX * sizeof(float);
+    if (indexed) bytes += list_ws_ints(make_params(d, true)) * sizeof(int);
+    return bytes;
+}
+
 int launch_bwd_mfma(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v, const int64_t* indices,
                     const void* w, const void* dout, const float* lse, void* dq, void* dk, void* dv, float* dw,
                     float* delta, hipStream_t s) {
-    return launch_bwd_generic(d, indexed, q, k, v, indices, w, dout, lse, dq, dk, dv, dw, delta, s);
+    if (!mfma_supported(d)) return GCA_ERR_UNSUPPORTED;
+    const Params p = make_params(d, indexed);
+    const int wb = d.w_dtype == GCA_BF16 ? 1 : 0;
+    if (d.D == 64) return launch_bwd_d<64>(p, q, k, v, indices, w, wb, dout, lse, dq, dk, dv, dw, delta, s);
+    return launch_bwd_d<128>(p, q, k, v, indices, w, wb, dout, lse, dq, dk, dv, dw, delta, s);
 }
-}
+
+}  // namespace gca

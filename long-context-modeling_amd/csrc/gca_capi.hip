@@ -69,7 +69,8 @@ int gca_fwd(const gca_desc* desc, const void* q, const void* k, const void* v, c
 
 size_t gca_bwd_workspace_bytes(const gca_desc* desc) {
     if (check_desc(desc, false) != GCA_OK) return 0;
-    return (size_t)desc->Z * desc->Hq * desc->K * desc->Q_CTX * sizeof(float);
+    const bool indexed = desc->N > 0 && desc->C > 0 && desc->Z % desc->N == 0;
+    return bwd_workspace_bytes(*desc, indexed);
 }
 
 int gca_bwd(const gca_desc* desc, const void* q, const void* k, const void* v, const void* weights,

@@ -86,4 +86,5 @@ int launch_lmk_score(const lmk_desc& d, const void* lq, const void* lk, void* sc
 int launch_lmk_topk(const lmk_desc& d, const void* scores, const void* noise, int64_t* indices, float* weights,
                     void* ws, size_t ws_bytes, hipStream_t s);
 size_t lmk_topk_ws_bytes(const lmk_desc& d);
+size_t bwd_workspace_bytes(const gca_desc& d, bool indexed);
 }  // namespace gca

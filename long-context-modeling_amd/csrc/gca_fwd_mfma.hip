@@ -20,15 +20,9 @@
 //                   column of a 4-key x 16-dim patch, i.e. the transposed access V needs.
 // The softmax denominator includes sm_n * exp2(-m) (sm_n virtual keys of logit 0 and value 0).
 // lse[z, h, j, row] = m + log2(l) in the log2-scaled domain, written when lse != NULL.
-#include "gca_common.h"
+#include "gca_mfma.h"
 
 namespace gca {
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-typedef __attribute__((ext_vector_type(4))) short s16x4;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 
 template <int D> struct FwdCfg {
     static constexpr int KSTRIDE = D * 2 + 16;   // bytes per K row in LDS: 16-byte reads of 8 rows hit distinct banks
@@ -37,20 +31,6 @@ template <int D> struct FwdCfg {
     static constexpr int VBYTES = 64 * VSTRIDE;
     static constexpr int BUF = KBYTES + VBYTES;
 };
-
-__device__ __forceinline__ bf16x8 lds_read_b128(const unsigned char* p) {
-    return *reinterpret_cast<const bf16x8*>(p);
-}
-
-__device__ __forceinline__ bf16x8 lds_read_tr_pair(const unsigned char* p0, const unsigned char* p1) {
-    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p0);
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p1);
-    union { s16x4 s[2]; bf16x8 v; } u;
-    u.s[0] = lo;
-    u.s[1] = hi;
-    return u.v;
-}
 
 template <int D, int GS, bool INDEXED>
 __global__ void __launch_bounds__(128 * GS)

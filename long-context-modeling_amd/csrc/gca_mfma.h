@@ -1,0 +1,75 @@
+// Register-level helpers shared by the gfx950 matrix-core kernels.
+//
+// v_mfma_f32_32x32x16_bf16 operand layout (lane = (n = lane % 32, h = lane / 32)):
+//   A: lane holds row n, reduction slots 8h .. 8h+7          B: lane holds column n, same slots
+//   C: lane holds column n; register r is row 8*(r/4) + 4*h + r%4
+// Only the pairing of slots between A and B matters for a product, so the kernels pick
+// the slot -> index map that lets one product's C registers be the next product's A operand:
+// for the 16-wide reduction step t, slots 0-3 are indices 16t + 4h + c and slots 4-7 are
+// 16t + 8 + 4h + c, which is the order C registers 8*(t%2) .. +7 of 32-row tile t/2 come in.
+//
+// LDS tiles are 64 rows of D bf16 without padding; the 16-byte pieces of a row are XOR-swizzled
+// with swz(row) so that the three access patterns used here are all bank-conflict free:
+// 16-byte writes of a row's pieces, 16-byte operand reads of 8 consecutive rows at one piece, and
+// ds_read_tr16_b64 patches of 4 consecutive rows x 32 bytes.
+#pragma once
+#include "gca_common.h"
+
+namespace gca {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+
+__device__ __forceinline__ int swz(int row) { return 2 * (row & 3) + ((row >> 2) & 1); }
+
+// byte offset of 16-byte piece `piece` of row `row` in a swizzled tile with RB bytes per row
+__device__ __forceinline__ int tile_off(int row, int piece, int RB) { return row * RB + ((piece ^ swz(row)) << 4); }
+
+__device__ __forceinline__ bf16x8 lds_read_b128(const unsigned char* p) {
+    return *reinterpret_cast<const bf16x8*>(p);
+}
+
+// Two transposed 4x16 patch reads: the lane gets, for its column, rows K0..K0+3 (p0) and K0+8..K0+11 (p1).
+__device__ __forceinline__ bf16x8 lds_read_tr_pair(const unsigned char* p0, const unsigned char* p1) {
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p0);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)p1);
+    union { s16x4 s[2]; bf16x8 v; } u;
+    u.s[0] = lo;
+    u.s[1] = hi;
+    return u.v;
+}
+
+// Per-lane constants of the transposed B-operand read of a swizzled [index][dim] tile:
+// reduction step t4 (16 indices), dim block db (32 dims).  Row = 16*t4 + 4h + (i16>>2) (+8 for the
+// second patch), 16-byte piece = 4*db + 2*dhalf + ((i16&3)>>1), 8-byte half = i16 & 1.
+struct TrLane {
+    int row0;     // 4h + (i16 >> 2)
+    int fsw;      // swz(row) -- the same for every t4 and for the +8 row
+    int piece0;   // 2*dhalf + ((i16 & 3) >> 1)
+    int half8;    // (i16 & 1) * 8
+    __device__ __forceinline__ explicit TrLane(int lane) {
+        const int i16 = lane & 15, h = lane >> 5, dhalf = (lane >> 4) & 1;
+        row0 = 4 * h + (i16 >> 2);
+        fsw = 2 * (i16 >> 2) + h;
+        piece0 = 2 * dhalf + ((i16 & 3) >> 1);
+        half8 = (i16 & 1) * 8;
+    }
+    __device__ __forceinline__ int off(int t4, int db, int RB) const {
+        return (16 * t4 + row0) * RB + (((4 * db + piece0) ^ fsw) << 4) + half8;
+    }
+};
+
+__device__ __forceinline__ float load_w(const void* w, int w_is_bf16, int64_t i) {
+    return w_is_bf16 ? bf16_bits_to_f(((const uint16_t*)w)[i]) : ((const float*)w)[i];
+}
+
+__device__ __forceinline__ uint16_t bf16_bits(float x) {
+    const __bf16 b = (__bf16)x;
+    return __builtin_bit_cast(uint16_t, b);
+}
+
+}  // namespace gca

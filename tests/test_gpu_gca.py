@@ -199,3 +199,34 @@ def test_indexed_equals_gathered(dtype):
     assert rel_err(wd.grad, w64.grad[:, :-1].reshape(-1, K)) <= tol
     o2 = gca_hip.gca_kv_cache_indexed(qd.detach(), ckd.detach(), cvd.detach(), idxd, wd.detach(), 1 / 8, 1.0)
     assert torch.equal(o2, o.detach())
+
+
+def test_indexed_hot_chunk_uses_segmented_lists():
+    # one cache chunk retrieved by every query chunk: its reference list is longer than one
+    # dkdv workgroup takes, so it is cut into segments whose partial sums are added atomically
+    import gca_hip
+    N, C, S, Hq, Hkv, d, K = 1, 41, 64, 2, 2, 64, 4
+    dtype = torch.bfloat16
+    ck = gen((N, C, S, Hkv * d), 20, 0.5, dtype)
+    cv = gen((N, C, S, Hkv * d), 21, 0.5, dtype)
+    g = torch.Generator().manual_seed(22)
+    idx = torch.randint(0, C, (N, C, K), generator=g)
+    idx[:, :, 0] = 0
+    w = torch.softmax(torch.rand(N, C, K, generator=g), -1)
+    q = gen((N * (C - 1), Hq, S, d), 23, 0.5, dtype)
+    do = gen((N * (C - 1), Hq, S, d), 24, 1.0, dtype)
+    ck64, cv64 = ck.double().requires_grad_(True), cv.double().requires_grad_(True)
+    q64, w64 = q.double().requires_grad_(True), w.double().requires_grad_(True)
+    kg, vg, wg = orc.gather_chunks(ck64, cv64, idx, w64, Hkv)
+    orc.gca_forward(q64, kg, vg, wg, 1 / 8, 0.0).backward(do.double())
+    qd, ckd, cvd = [t.cuda().requires_grad_(True) for t in (q, ck, cv)]
+    wd = w[:, :-1].reshape(-1, K).contiguous().cuda().requires_grad_(True)
+    idxd = idx[:, :-1].reshape(-1, K).contiguous().cuda()
+    gca_hip.attention_indexed(qd, ckd, cvd, idxd, wd, 1 / 8, 0.0).backward(do.cuda())
+    tol = TOL[dtype]
+    assert rel_err(qd.grad, q64.grad) <= tol
+    assert rel_err(ckd.grad, ck64.grad) <= tol
+    assert rel_err(cvd.grad, cv64.grad) <= tol
+    assert rel_err(wd.grad, w64.grad[:, :-1].reshape(-1, K)) <= tol
+    never = torch.ones(C, dtype=torch.bool); never[idx[0, :-1].unique()] = False
+    assert ckd.grad[0, never].abs().max() == 0          # chunks nobody retrieved get zero gradient
