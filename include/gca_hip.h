@@ -53,6 +53,15 @@ enum gca_status {
  * when the shape does not qualify). */
 enum gca_path { GCA_PATH_AUTO = 0, GCA_PATH_GENERIC = 1, GCA_PATH_MFMA = 2 };
 
+/* gca_bwd / gca_bwd_indexed are several launches.  desc.stages selects which of them run
+ * (0 = all); a profiler or benchmark can time one stage with events around the call.  Running a
+ * later stage alone needs the buffers an earlier stage fills (delta in the workspace). */
+enum gca_stage {
+    GCA_STAGE_DQ = 1,      /* dq and the per-chunk row sums delta */
+    GCA_STAGE_DKDV = 2,    /* reference lists (indexed form) and dk, dv */
+    GCA_STAGE_DW = 4       /* dw from delta */
+};
+
 typedef struct gca_desc {
     int32_t dtype;      /* gca_dtype of q, k, v, o and their gradients */
     int32_t w_dtype;    /* gca_dtype of weights */
@@ -66,7 +75,7 @@ typedef struct gca_desc {
     float sm_scale;     /* multiplies q.k before the softmax */
     float sm_n;         /* softmax denominator offset: P = exp(s) / (sm_n + sum exp(s)); 0 = plain */
     int32_t path;       /* gca_path */
-    int32_t reserved;
+    int32_t stages;     /* bitmask of gca_stage for the backward entry points; 0 = all */
     int64_t N;          /* indexed entry points: sequences in the cache (Z % N == 0) */
     int64_t C;          /* indexed entry points: chunks per sequence in the cache */
 } gca_desc;
@@ -93,7 +102,8 @@ const char* gca_strerror(int status);
 int gca_fwd(const gca_desc* desc, const void* q, const void* k, const void* v, const void* weights,
             void* o, float* lse, void* stream);
 
-/* Bytes of scratch gca_bwd needs (the per-chunk row sums D_j, (Z, Hq, K, Q_CTX) floats). */
+/* Bytes of scratch the backward needs: the per-chunk row sums D_j ((Z, Hq, K, Q_CTX) floats) and,
+ * when desc.N and desc.C are set (gca_bwd_indexed), the reference lists of the cache chunks. */
 size_t gca_bwd_workspace_bytes(const gca_desc* desc);
 
 /* Backward on gathered K/V: dq, dk, dv in T, dw in float.

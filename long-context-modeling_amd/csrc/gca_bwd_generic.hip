@@ -248,9 +248,11 @@ static int launch_d(const Params& p, const void* q, const void* k, const void* v
     const int nkb = (p.K_CTX + 31) / 32;
     const int64_t b2 = p.Z * p.Hkv * p.K * nkb;
     if (b1 <= 0 || b1 > 0x7fffffffLL || b2 <= 0 || b2 > 0x7fffffffLL) return GCA_ERR_SHAPE;
-    hipLaunchKernelGGL((gca_bwd_dq_generic_kernel<T, WT, D>), dim3((unsigned)b1), dim3(256), 0, s, p,
-                       (const T*)q, (const T*)k, (const T*)v, idx, (const WT*)w, (const T*)dout, lse, (T*)dq, delta);
+    if (p.stages & GCA_STAGE_DQ)
+        hipLaunchKernelGGL((gca_bwd_dq_generic_kernel<T, WT, D>), dim3((unsigned)b1), dim3(256), 0, s, p,
+                           (const T*)q, (const T*)k, (const T*)v, idx, (const WT*)w, (const T*)dout, lse, (T*)dq, delta);
     if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
+    if (!(p.stages & GCA_STAGE_DKDV)) return (p.stages & GCA_STAGE_DW) ? launch_dw(p, delta, dw, s) : GCA_OK;
     if (p.indexed)
         hipLaunchKernelGGL((gca_bwd_dkdv_generic_kernel<T, WT, D, true>), dim3((unsigned)b2), dim3(256), 0, s, p,
                            (const T*)q, (const T*)k, (const T*)v, idx, (const WT*)w, (const T*)dout, lse, delta, dk, dv);
@@ -258,7 +260,7 @@ static int launch_d(const Params& p, const void* q, const void* k, const void* v
         hipLaunchKernelGGL((gca_bwd_dkdv_generic_kernel<T, WT, D, false>), dim3((unsigned)b2), dim3(256), 0, s, p,
                            (const T*)q, (const T*)k, (const T*)v, idx, (const WT*)w, (const T*)dout, lse, delta, dk, dv);
     if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
-    return launch_dw(p, delta, dw, s);
+    return (p.stages & GCA_STAGE_DW) ? launch_dw(p, delta, dw, s) : GCA_OK;
 }
 
 template <typename T, typename WT>

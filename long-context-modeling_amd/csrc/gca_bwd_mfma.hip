@@ -536,11 +536,14 @@ template <int D>
 static int launch_bwd_d(const Params& p, const void* q, const void* k, const void* v, const int64_t* idx, const void* w,
                         int wb, const void* dout, const float* lse, void* dq, void* dk, void* dv, float* dw,
                         float* delta, hipStream_t s) {
-    int rc;
-    if (p.G % 4 == 0) rc = launch_dq_gs<D, 4>(p, q, k, v, idx, w, wb, dout, lse, dq, delta, s);
-    else if (p.G % 2 == 0) rc = launch_dq_gs<D, 2>(p, q, k, v, idx, w, wb, dout, lse, dq, delta, s);
-    else rc = launch_dq_gs<D, 1>(p, q, k, v, idx, w, wb, dout, lse, dq, delta, s);
-    if (rc != GCA_OK) return rc;
+    int rc = GCA_OK;
+    if (p.stages & GCA_STAGE_DQ) {
+        if (p.G % 4 == 0) rc = launch_dq_gs<D, 4>(p, q, k, v, idx, w, wb, dout, lse, dq, delta, s);
+        else if (p.G % 2 == 0) rc = launch_dq_gs<D, 2>(p, q, k, v, idx, w, wb, dout, lse, dq, delta, s);
+        else rc = launch_dq_gs<D, 1>(p, q, k, v, idx, w, wb, dout, lse, dq, delta, s);
+        if (rc != GCA_OK) return rc;
+    }
+    if (!(p.stages & GCA_STAGE_DKDV)) return (p.stages & GCA_STAGE_DW) ? launch_dw(p, delta, dw, s) : GCA_OK;
 
     ListWs ws = {};
     if (p.indexed) {
@@ -566,7 +569,7 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
                            dk, dv, ws);
     }
     if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
-    return launch_dw(p, delta, dw, s);
+    return (p.stages & GCA_STAGE_DW) ? launch_dw(p, delta, dw, s) : GCA_OK;
 }
 
 size_t bwd_workspace_bytes(const gca_desc& d, bool indexed) {

@@ -37,6 +37,7 @@ struct Params {
     // indexed variants
     int64_t N, C, zpn;   // zpn = Z / N rows per sequence
     int32_t indexed;
+    int32_t stages;      // gca_stage bitmask, never 0 here
 };
 
 inline Params make_params(const gca_desc& d, bool indexed) {
@@ -47,6 +48,7 @@ inline Params make_params(const gca_desc& d, bool indexed) {
     p.N = indexed ? d.N : 1; p.C = indexed ? d.C : 1;
     p.zpn = indexed ? d.Z / d.N : d.Z;
     p.indexed = indexed ? 1 : 0;
+    p.stages = d.stages == 0 ? 7 : d.stages;
     return p;
 }
 

@@ -29,7 +29,7 @@ class GcaDesc(ctypes.Structure):
         ("Hq", ctypes.c_int32), ("Hkv", ctypes.c_int32), ("K", ctypes.c_int32),
         ("Q_CTX", ctypes.c_int32), ("K_CTX", ctypes.c_int32), ("D", ctypes.c_int32),
         ("sm_scale", ctypes.c_float), ("sm_n", ctypes.c_float),
-        ("path", ctypes.c_int32), ("reserved", ctypes.c_int32),
+        ("path", ctypes.c_int32), ("stages", ctypes.c_int32),
         ("N", ctypes.c_int64), ("C", ctypes.c_int64),
     ]
 

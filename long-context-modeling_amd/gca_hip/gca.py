@@ -61,7 +61,7 @@ def _desc(q, K, K_CTX, Hkv, weights, sm_scale, sm_n, path=None, N=0, C=0):
     Z, Hq, Q_CTX, D = q.shape
     return _lib.GcaDesc(
         dtype=_DT[q.dtype], w_dtype=_DT[weights.dtype], Z=Z, Hq=Hq, Hkv=Hkv, K=K, Q_CTX=Q_CTX, K_CTX=K_CTX, D=D,
-        sm_scale=float(sm_scale), sm_n=float(sm_n), path=_PATHS[path or kernel_path], reserved=0, N=N, C=C)
+        sm_scale=float(sm_scale), sm_n=float(sm_n), path=_PATHS[path or kernel_path], stages=0, N=N, C=C)
 
 
 def _forward(q, k, v, weights, sm_scale, sm_n, want_lse, path=None):

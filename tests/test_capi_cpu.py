@@ -34,7 +34,7 @@ def test_struct_layout_matches_header():
 
 def _desc(**kw):
     base = dict(dtype=1, w_dtype=0, Z=2, Hq=4, Hkv=2, K=2, Q_CTX=64, K_CTX=64, D=64, sm_scale=0.125, sm_n=0.0,
-                path=0, reserved=0, N=0, C=0)
+                path=0, stages=0, N=0, C=0)
     base.update(kw)
     return _lib.GcaDesc(**base)
 
