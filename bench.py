@@ -71,8 +71,7 @@ def kernel_times(torch, q, ck, cv, idx, w, do, sm_scale, sm_n, iters):
     o = torch.empty_like(q)
     lse = torch.empty((Z, H, K, S), device=dev, dtype=torch.float32)
     dq = torch.empty_like(q)
-    dkc = torch.zeros(ck.shape, device=dev, dtype=torch.float32)
-    dvc = torch.zeros(cv.shape, device=dev, dtype=torch.float32)
+    dkc, dvc = torch.empty_like(ck), torch.empty_like(cv)
     dw = torch.empty((Z, K), device=dev, dtype=torch.float32)
     stream = _stream(dev)
 

@@ -120,13 +120,13 @@ int gca_bwd(const gca_desc* desc, const void* q, const void* k, const void* v, c
 int gca_fwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, const void* v_cache,
                     const int64_t* indices, const void* weights, void* o, float* lse, void* stream);
 
-/* Backward of gca_fwd_indexed.  dk_cache / dv_cache are FLOAT buffers of the cache's
- * shape (N, C, K_CTX, Hkv*D) that the caller has zeroed; gradients of chunks retrieved
- * by several query chunks are summed into them (the index_put_(accumulate=True) that
- * autograd runs for model/DRT.py:198-199). */
+/* Backward of gca_fwd_indexed.  dk_cache / dv_cache have the cache's shape (N, C, K_CTX, Hkv*D)
+ * and element type T and are written completely by the call (zeros for chunks nobody retrieved);
+ * gradients of a chunk retrieved by several query chunks are summed, in a fixed order, without
+ * atomics (the index_put_(accumulate=True) that autograd runs for model/DRT.py:198-199). */
 int gca_bwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, const void* v_cache,
                     const int64_t* indices, const void* weights, const void* dout, const float* lse,
-                    void* dq, float* dk_cache, float* dv_cache, float* dw,
+                    void* dq, void* dk_cache, void* dv_cache, float* dw,
                     void* workspace, size_t workspace_bytes, void* stream);
 
 /* scores[n, c, e] = <lmk_q[n, c, :], lmk_k[n, e, :]> / sqrt(hidden_size), -inf where masked.

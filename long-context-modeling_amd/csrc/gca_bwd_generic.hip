@@ -1,21 +1,25 @@
 // Generic GCA backward: fp32 arithmetic on the vector ALUs for any supported shape and
 // element type (the fp32 path and the fallback for shapes the MFMA kernels do not take).
 //
-// Three launches, no atomics in the gathered form:
+// Three launches (plus the list build in the indexed form), no atomics:
 //   1. dq kernel   one workgroup = 32 query rows of one (z, query head).  Per retrieved chunk
 //                  it makes two passes over the key tiles: the first builds
 //                  D_j = rowsum(P_j * dP_j) (stored to `delta`), the second forms
 //                  dS = w P (dP - D_j) and accumulates dQ += dS K.
-//   2. dkdv kernel one workgroup = 32 key rows of one (z, kv head, retrieved chunk); loops over
-//                  the query heads of the group and their rows, using lse and delta.
-//                  Gathered form: writes dk, dv in T.  Indexed form: atomically adds into the
-//                  float cache-shaped gradient buffers (several query chunks may have
-//                  retrieved the same cache chunk).
+//   2. dkdv kernel one workgroup = 32 key rows of one key/value tile; loops over the (z, j) that
+//                  read the tile, the query heads of the group and their rows, using lse and delta.
+//                  Gathered form: the tile is slot (z, kv head, j), read by that (z, j) only.
+//                  Indexed form: the tile is a cache chunk and the walk follows the chunk's
+//                  reference list (built on the device), so dk/dv are written once, in T, in
+//                  the cache's layout, with a fixed summation order.
 //   3. dw kernel   dw[z, j] = sum over heads and rows of delta.
 // Same lane mapping as the generic forward: 8 lanes share a row and own D/8 dims each.
 #include "gca_common.h"
+#include "gca_lists.h"
 
 namespace gca {
+
+constexpr int GENERIC_SEG_MAX = 1 << 30;
 
 template <typename T, typename WT, int D>
 __global__ void __launch_bounds__(256)
@@ -109,7 +113,7 @@ __global__ void __launch_bounds__(256)
 gca_bwd_dkdv_generic_kernel(Params p, const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
                             const int64_t* __restrict__ indices, const WT* __restrict__ w,
                             const T* __restrict__ dout, const float* __restrict__ lse,
-                            const float* __restrict__ delta, void* __restrict__ dk_out, void* __restrict__ dv_out) {
+                            const float* __restrict__ delta, T* __restrict__ dk_out, T* __restrict__ dv_out, ListWs ws) {
     constexpr int TPR = 8, KB = 32, DPT = D / TPR;
     constexpr int QT = (D >= 256) ? 16 : 32;
     __shared__ float sQ[QT * D];
@@ -122,15 +126,30 @@ gca_bwd_dkdv_generic_kernel(Params p, const T* __restrict__ q, const T* __restri
     const int nkb = (p.K_CTX + KB - 1) / KB;
     int64_t bid = blockIdx.x;
     const int kb = (int)(bid % nkb); bid /= nkb;
-    const int j = (int)(bid % p.K); bid /= p.K;
-    const int hk = (int)(bid % p.Hkv);
-    const int64_t z = bid / p.Hkv;
     const int krow = kb * KB + r;
     const bool row_ok = krow < p.K_CTX;
-
-    int64_t rs;
-    const T* kj = chunk_base(p, k, indices, z, hk, j, rs);
-    const T* vj = chunk_base(p, v, indices, z, hk, j, rs);
+    // gathered: the tile is slot (z, hk, j) and is visited by that one (z, j).
+    // indexed: the tile is cache chunk cc and is visited by every reference in the chunk's list.
+    int hk, nref, list0 = 0;
+    int64_t gz = 0, rs, tile_off;
+    int gj = 0;
+    if (INDEXED) {
+        hk = (int)(bid % p.Hkv);
+        const int64_t cc = bid / p.Hkv;
+        nref = ws.count[cc];
+        list0 = ws.start[cc];
+        rs = (int64_t)p.Hkv * D;
+        tile_off = cc * p.K_CTX * rs + (int64_t)hk * D;
+    } else {
+        gj = (int)(bid % p.K); bid /= p.K;
+        hk = (int)(bid % p.Hkv);
+        gz = bid / p.Hkv;
+        nref = 1;
+        rs = D;
+        tile_off = (((gz * p.Hkv + hk) * p.K + gj) * (int64_t)p.K_CTX) * D;
+    }
+    const T* kj = k + tile_off;
+    const T* vj = v + tile_off;
     float kreg[DPT], vreg[DPT], dkacc[DPT], dvacc[DPT];
 #pragma unroll
     for (int i = 0; i < DPT; ++i) { kreg[i] = 0.f; vreg[i] = 0.f; dkacc[i] = 0.f; dvacc[i] = 0.f; }
@@ -142,8 +161,16 @@ gca_bwd_dkdv_generic_kernel(Params p, const T* __restrict__ q, const T* __restri
         }
     }
     const float c = p.sm_scale * LOG2E;
-    const float wj = to_f(w[z * p.K + j]);
 
+    for (int ri = 0; ri < nref; ++ri) {
+    int64_t z = gz;
+    int j = gj;
+    if (INDEXED) {
+        const int ref = ws.refs[list0 + ri];
+        z = ref / p.K;
+        j = ref % p.K;
+    }
+    const float wj = to_f(w[z * p.K + j]);
     for (int g = 0; g < p.G; ++g) {
         const int h = hk * p.G + g;
         const int64_t qbase = (z * p.Hq + h) * (int64_t)p.Q_CTX;
@@ -189,28 +216,13 @@ gca_bwd_dkdv_generic_kernel(Params p, const T* __restrict__ q, const T* __restri
             }
         }
     }
+    }
     if (row_ok) {
-        if (INDEXED) {
-            const int64_t n = z / p.zpn;
-            int64_t cidx = indices[z * p.K + j];
-            cidx = cidx < 0 ? 0 : (cidx >= p.C ? p.C - 1 : cidx);
-            const int64_t off = (((n * p.C + cidx) * p.K_CTX + krow) * p.Hkv + hk) * (int64_t)D + t * DPT;
-            float* dkc = (float*)dk_out + off;
-            float* dvc = (float*)dv_out + off;
+        const int64_t off = tile_off + (int64_t)krow * rs + t * DPT;
 #pragma unroll
-            for (int i = 0; i < DPT; ++i) {
-                atomicAdd(dkc + i, dkacc[i] * p.sm_scale);
-                atomicAdd(dvc + i, dvacc[i]);
-            }
-        } else {
-            const int64_t off = ((((z * p.Hkv + hk) * p.K + j) * (int64_t)p.K_CTX) + krow) * D + t * DPT;
-            T* dkp = (T*)dk_out + off;
-            T* dvp = (T*)dv_out + off;
-#pragma unroll
-            for (int i = 0; i < DPT; ++i) {
-                dkp[i] = from_f<T>(dkacc[i] * p.sm_scale);
-                dvp[i] = from_f<T>(dvacc[i]);
-            }
+        for (int i = 0; i < DPT; ++i) {
+            dk_out[off + i] = from_f<T>(dkacc[i] * p.sm_scale);
+            dv_out[off + i] = from_f<T>(dvacc[i]);
         }
     }
 }
@@ -246,19 +258,27 @@ static int launch_d(const Params& p, const void* q, const void* k, const void* v
     const int nqb = (p.Q_CTX + 31) / 32;
     const int64_t b1 = p.Z * p.Hq * nqb;
     const int nkb = (p.K_CTX + 31) / 32;
-    const int64_t b2 = p.Z * p.Hkv * p.K * nkb;
+    const int64_t b2 = (p.indexed ? p.N * p.C * p.Hkv : p.Z * p.Hkv * p.K) * nkb;
     if (b1 <= 0 || b1 > 0x7fffffffLL || b2 <= 0 || b2 > 0x7fffffffLL) return GCA_ERR_SHAPE;
     if (p.stages & GCA_STAGE_DQ)
         hipLaunchKernelGGL((gca_bwd_dq_generic_kernel<T, WT, D>), dim3((unsigned)b1), dim3(256), 0, s, p,
                            (const T*)q, (const T*)k, (const T*)v, idx, (const WT*)w, (const T*)dout, lse, (T*)dq, delta);
     if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
     if (!(p.stages & GCA_STAGE_DKDV)) return (p.stages & GCA_STAGE_DW) ? launch_dw(p, delta, dw, s) : GCA_OK;
-    if (p.indexed)
+    ListWs ws = {};
+    if (p.indexed) {
+        // every chunk's list is walked whole by one workgroup here: no segments, no partial slots
+        ws = list_carve(p, GENERIC_SEG_MAX, (char*)delta + delta_bytes(p));
+        const int rc = list_build(p, GENERIC_SEG_MAX, idx, ws, s);
+        if (rc != GCA_OK) return rc;
         hipLaunchKernelGGL((gca_bwd_dkdv_generic_kernel<T, WT, D, true>), dim3((unsigned)b2), dim3(256), 0, s, p,
-                           (const T*)q, (const T*)k, (const T*)v, idx, (const WT*)w, (const T*)dout, lse, delta, dk, dv);
-    else
+                           (const T*)q, (const T*)k, (const T*)v, idx, (const WT*)w, (const T*)dout, lse, delta,
+                           (T*)dk, (T*)dv, ws);
+    } else {
         hipLaunchKernelGGL((gca_bwd_dkdv_generic_kernel<T, WT, D, false>), dim3((unsigned)b2), dim3(256), 0, s, p,
-                           (const T*)q, (const T*)k, (const T*)v, idx, (const WT*)w, (const T*)dout, lse, delta, dk, dv);
+                           (const T*)q, (const T*)k, (const T*)v, idx, (const WT*)w, (const T*)dout, lse, delta,
+                           (T*)dk, (T*)dv, ws);
+    }
     if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
     return (p.stages & GCA_STAGE_DW) ? launch_dw(p, delta, dw, s) : GCA_OK;
 }

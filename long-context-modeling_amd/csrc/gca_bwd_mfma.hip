@@ -19,16 +19,17 @@
 //      dV += P~^T dO,  dK += dS^T Q      dO and Q read transposed from LDS
 //    Gathered form: the tile is slot (z, kv head, j) and the walk is the G heads of the group; dk/dv
 //    are written in bf16.  Indexed form: the tile is a chunk of the cache and the walk follows a
-//    reference list built on the device (count -> scan -> fill, every list ordered by (z, j), no
-//    atomics, so the summation order is fixed).  Lists longer than SEG_MAX are cut into segments handled by
-//    separate workgroups; only those chunks use float atomics, all others store directly.
+//    reference list built on the device (every list ordered by (z, j), no atomics, so the summation
+//    order is fixed); dk/dv come out in bf16 in the cache's own layout, every element written once.
+//    Lists longer than SEG_MAX are cut into segments handled by separate workgroups that write float
+//    partial tiles; a small reduce launch adds those up in segment order.
 //
 // dw[z, j] = sum over heads and rows of delta (shared launch_dw).
 #include "gca_mfma.h"
+#include "gca_lists.h"
 
 namespace gca {
 
-int launch_dw(const Params& p, const float* delta, float* dw, hipStream_t s);
 
 constexpr int SEG_MAX = 16;   // references per dkdv workgroup in the indexed form
 
@@ -191,110 +192,6 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
         }
 }
 
-// ------------------------------------------------------------------------------------------- lists
-
-// Reference lists of the indexed form.  Chunk cc = n*C + c of the cache is referenced by
-// ref = z*K + j whenever indices[z, j] == c and z belongs to sequence n.
-struct ListWs {
-    int* count;      // [NC]      references per chunk
-    int* start;      // [NC]      first slot of the chunk's list in refs
-    int* seg_base;   // [NC]      first segment of the chunk
-    int* nseg;       // [1]       total segments
-    int* refs;       // [Z*K]     reference ids, chunk by chunk, each list ascending
-    int* seg_chunk;  // [bound]   chunk of a segment
-    int* seg_start;  // [bound]   first slot in refs
-    int* seg_len;    // [bound]   references in the segment (<= SEG_MAX)
-    int* seg_multi;  // [bound]   1 if the chunk has more than one segment
-};
-
-static inline int64_t seg_bound(const Params& p) { return p.N * p.C + (p.Z * p.K + SEG_MAX - 1) / SEG_MAX; }
-
-static inline size_t list_ws_ints(const Params& p) {
-    return (size_t)(3 * p.N * p.C + 4 + p.Z * p.K + 4 * seg_bound(p));
-}
-
-static ListWs carve_list_ws(const Params& p, int* base) {
-    ListWs ws;
-    const int64_t NC = p.N * p.C, sb = seg_bound(p);
-    ws.count = base; base += NC;
-    ws.start = base; base += NC;
-    ws.seg_base = base; base += NC;
-    ws.nseg = base; base += 4;
-    ws.refs = base; base += p.Z * p.K;
-    ws.seg_chunk = base; base += sb;
-    ws.seg_start = base; base += sb;
-    ws.seg_len = base; base += sb;
-    ws.seg_multi = base;
-    return ws;
-}
-
-__device__ __forceinline__ int64_t clamp_idx(int64_t c, int64_t C) { return c < 0 ? 0 : (c >= C ? C - 1 : c); }
-
-__global__ void __launch_bounds__(256)
-gca_bwd_list_count_kernel(Params p, const int64_t* __restrict__ indices, ListWs ws) {
-    const int64_t cc = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (cc >= p.N * p.C) return;
-    const int64_t n = cc / p.C, c = cc % p.C;
-    const int64_t r0 = n * p.zpn * p.K, r1 = r0 + p.zpn * p.K;
-    int cnt = 0;
-    for (int64_t r = r0; r < r1; ++r) cnt += (clamp_idx(indices[r], p.C) == c) ? 1 : 0;
-    ws.count[cc] = cnt;
-}
-
-// one workgroup: exclusive scans of the counts (list starts) and of the segment counts
-__global__ void __launch_bounds__(1024)
-gca_bwd_list_scan_kernel(Params p, ListWs ws) {
-    __shared__ int s_cnt[1024], s_seg[1024];
-    __shared__ int carry_cnt, carry_seg;
-    const int tid = threadIdx.x;
-    const int64_t NC = p.N * p.C;
-    if (tid == 0) { carry_cnt = 0; carry_seg = 0; }
-    __syncthreads();
-    for (int64_t base = 0; base < NC; base += 1024) {
-        const int64_t cc = base + tid;
-        const int cnt = cc < NC ? ws.count[cc] : 0;
-        const int sg = (cnt + SEG_MAX - 1) / SEG_MAX;
-        s_cnt[tid] = cnt;
-        s_seg[tid] = sg;
-        __syncthreads();
-        for (int off = 1; off < 1024; off <<= 1) {
-            const int a = tid >= off ? s_cnt[tid - off] : 0;
-            const int b = tid >= off ? s_seg[tid - off] : 0;
-            __syncthreads();
-            s_cnt[tid] += a;
-            s_seg[tid] += b;
-            __syncthreads();
-        }
-        if (cc < NC) {
-            ws.start[cc] = carry_cnt + s_cnt[tid] - cnt;
-            ws.seg_base[cc] = carry_seg + s_seg[tid] - sg;
-        }
-        __syncthreads();
-        if (tid == 1023) { carry_cnt += s_cnt[1023]; carry_seg += s_seg[1023]; }
-        __syncthreads();
-    }
-    if (tid == 0) ws.nseg[0] = carry_seg;
-}
-
-__global__ void __launch_bounds__(256)
-gca_bwd_list_fill_kernel(Params p, const int64_t* __restrict__ indices, ListWs ws) {
-    const int64_t cc = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (cc >= p.N * p.C) return;
-    const int64_t n = cc / p.C, c = cc % p.C;
-    const int64_t r0 = n * p.zpn * p.K, r1 = r0 + p.zpn * p.K;
-    const int start = ws.start[cc], cnt = ws.count[cc];
-    int kfill = 0;
-    for (int64_t r = r0; r < r1 && kfill < cnt; ++r)
-        if (clamp_idx(indices[r], p.C) == c) ws.refs[start + kfill++] = (int)r;
-    const int sg = (cnt + SEG_MAX - 1) / SEG_MAX, sb = ws.seg_base[cc];
-    for (int s = 0; s < sg; ++s) {
-        ws.seg_chunk[sb + s] = (int)cc;
-        ws.seg_start[sb + s] = start + s * SEG_MAX;
-        ws.seg_len[sb + s] = min(SEG_MAX, cnt - s * SEG_MAX);
-        ws.seg_multi[sb + s] = sg > 1 ? 1 : 0;
-    }
-}
-
 // ------------------------------------------------------------------------------------------- dkdv
 
 template <int D, bool INDEXED>
@@ -317,7 +214,7 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
     const int n = lane & 31, h = lane >> 5;
 
     // ---- which tile, which walk
-    int hk, nunits, list0 = 0, multi = 0;
+    int hk, nunits, list0 = 0, slot = -1;
     int64_t gz = 0;          // gathered: the single (z, j)
     int gj = 0;
     const uint16_t* kt;
@@ -330,11 +227,20 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
         const int64_t cc = ws.seg_chunk[seg];
         list0 = ws.seg_start[seg];
         nunits = ws.seg_len[seg] * p.G * (p.Q_CTX / 64);
-        multi = ws.seg_multi[seg];
+        slot = ws.seg_slot[seg];
         rs = (int64_t)p.Hkv * D;
         out_off = cc * p.K_CTX * rs + (int64_t)hk * D;
         kt = k + out_off;
         vt = v + out_off;
+        if (nunits == 0) {
+            // nobody retrieved this chunk: its gradient is zero
+            for (int i = tid; i < 64 * D; i += NT) {
+                const int64_t off = out_off + (int64_t)(i / D) * rs + (i % D);
+                ((uint16_t*)dk_out)[off] = 0;
+                ((uint16_t*)dv_out)[off] = 0;
+            }
+            return;
+        }
     } else {
         int64_t bid = blockIdx.x;
         gj = (int)(bid % p.K); bid /= p.K;
@@ -499,19 +405,40 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
         for (int r = 0; r < 16; ++r) {
             const int row = 32 * kbw + 8 * (r >> 2) + 4 * h + (r & 3);
             const int64_t off = out_off + (int64_t)row * rs + 32 * db + n;
-            if (INDEXED) {
-                if (multi) {
-                    atomicAdd((float*)dk_out + off, dkacc[db][r]);
-                    atomicAdd((float*)dv_out + off, dvacc[db][r]);
-                } else {
-                    ((float*)dk_out)[off] = dkacc[db][r];
-                    ((float*)dv_out)[off] = dvacc[db][r];
-                }
+            if (INDEXED && slot >= 0) {
+                float* part = ws.partials + ((int64_t)slot * p.Hkv + hk) * 2 * (64 * D) + row * D + 32 * db + n;
+                part[0] = dkacc[db][r];
+                part[64 * D] = dvacc[db][r];
             } else {
                 ((uint16_t*)dk_out)[off] = bf16_bits(dkacc[db][r]);
                 ((uint16_t*)dv_out)[off] = bf16_bits(dvacc[db][r]);
             }
         }
+}
+
+// Chunks whose list was cut into several segments: add the float partial tiles in segment order.
+// grid = NC * Hkv workgroups; those of single-segment chunks return at once.
+template <int D>
+__global__ void __launch_bounds__(256)
+gca_bwd_dkdv_reduce_kernel(Params p, int seg_max, uint16_t* __restrict__ dk_out, uint16_t* __restrict__ dv_out, ListWs ws) {
+    const int64_t cc = blockIdx.x / p.Hkv;
+    const int hk = blockIdx.x % p.Hkv;
+    const int sg = (ws.count[cc] + seg_max - 1) / seg_max;
+    if (sg <= 1) return;
+    const int slot0 = ws.slot_base[cc];
+    const int64_t rs = (int64_t)p.Hkv * D;
+    const int64_t out_off = cc * p.K_CTX * rs + (int64_t)hk * D;
+    for (int i = threadIdx.x; i < 64 * D; i += 256) {
+        float ak = 0.f, av = 0.f;
+        for (int s = 0; s < sg; ++s) {
+            const float* part = ws.partials + ((int64_t)(slot0 + s) * p.Hkv + hk) * 2 * (64 * D) + i;
+            ak += part[0];
+            av += part[64 * D];
+        }
+        const int64_t off = out_off + (int64_t)(i / D) * rs + (i % D);
+        dk_out[off] = bf16_bits(ak);
+        dv_out[off] = bf16_bits(av);
+    }
 }
 
 // ------------------------------------------------------------------------------------------- launch
@@ -548,19 +475,15 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
     ListWs ws = {};
     if (p.indexed) {
         // the list workspace follows delta
-        int* base = (int*)(delta + (size_t)p.Z * p.Hq * p.K * p.Q_CTX);
-        ws = carve_list_ws(p, base);
-        const int64_t NC = p.N * p.C;
-        const unsigned nb = (unsigned)((NC + 255) / 256);
-        hipLaunchKernelGGL(gca_bwd_list_count_kernel, dim3(nb), dim3(256), 0, s, p, idx, ws);
-        hipLaunchKernelGGL(gca_bwd_list_scan_kernel, dim3(1), dim3(1024), 0, s, p, ws);
-        hipLaunchKernelGGL(gca_bwd_list_fill_kernel, dim3(nb), dim3(256), 0, s, p, idx, ws);
-        if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
-        const int64_t blocks = seg_bound(p) * p.Hkv;
+        ws = list_carve(p, SEG_MAX, (char*)delta + delta_bytes(p));
+        if ((rc = list_build(p, SEG_MAX, idx, ws, s)) != GCA_OK) return rc;
+        const int64_t blocks = list_seg_bound(p, SEG_MAX) * p.Hkv;
         if (blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
         hipLaunchKernelGGL((gca_bwd_dkdv_mfma_kernel<D, true>), dim3((unsigned)blocks), dim3(128), 0, s, p,
                            (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse, delta,
                            dk, dv, ws);
+        hipLaunchKernelGGL((gca_bwd_dkdv_reduce_kernel<D>), dim3((unsigned)(p.N * p.C * p.Hkv)), dim3(256), 0, s, p, SEG_MAX,
+                           (uint16_t*)dk, (uint16_t*)dv, ws);
     } else {
         const int64_t blocks = p.Z * p.Hkv * p.K;
         if (blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
@@ -573,8 +496,9 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
 }
 
 size_t bwd_workspace_bytes(const gca_desc& d, bool indexed) {
-    size_t bytes = (size_t)d.Z * d.Hq * d.K * d.Q_CTX * sizeof(float);
-    if (indexed) bytes += list_ws_ints(make_params(d, true)) * sizeof(int);
+    const Params p = make_params(d, indexed);
+    size_t bytes = delta_bytes(p);
+    if (indexed) bytes += list_ws_bytes(p, SEG_MAX);
     return bytes;
 }
 

@@ -103,7 +103,7 @@ int gca_fwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, co
 
 int gca_bwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, const void* v_cache,
                     const int64_t* indices, const void* weights, const void* dout, const float* lse,
-                    void* dq, float* dk_cache, float* dv_cache, float* dw,
+                    void* dq, void* dk_cache, void* dv_cache, float* dw,
                     void* workspace, size_t workspace_bytes, void* stream) {
     int rc = check_desc(desc, true);
     if (rc != GCA_OK) return rc;

@@ -89,4 +89,9 @@ int launch_lmk_topk(const lmk_desc& d, const void* scores, const void* noise, in
                     void* ws, size_t ws_bytes, hipStream_t s);
 size_t lmk_topk_ws_bytes(const lmk_desc& d);
 size_t bwd_workspace_bytes(const gca_desc& d, bool indexed);
+int launch_dw(const Params& p, const float* delta, float* dw, hipStream_t s);
+// bytes of the per-chunk row sums D_j at the start of the backward workspace (256-byte multiple)
+inline size_t delta_bytes(const Params& p) {
+    return ((size_t)p.Z * p.Hq * p.K * p.Q_CTX * sizeof(float) + 255) / 256 * 256;
+}
 }  // namespace gca

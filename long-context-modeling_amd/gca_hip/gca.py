@@ -159,8 +159,7 @@ class _AttentionIndexed(torch.autograd.Function):
         N, C, K_CTX, Dm = k_cache.shape
         Hkv, K = Dm // q.shape[-1], indices.shape[1]
         dq = torch.empty_like(q)
-        dkc = torch.zeros(k_cache.shape, device=q.device, dtype=torch.float32)
-        dvc = torch.zeros(v_cache.shape, device=q.device, dtype=torch.float32)
+        dkc, dvc = torch.empty_like(k_cache), torch.empty_like(v_cache)
         dw = torch.empty(weights.shape, device=q.device, dtype=torch.float32)
         desc = _desc(q, K, K_CTX, Hkv, weights, ctx.sm_scale, ctx.sm_n, N=N, C=C)
         with torch.cuda.device(q.device):
@@ -171,7 +170,7 @@ class _AttentionIndexed(torch.autograd.Function):
                                    _ptr(weights), _ptr(do), _ptr(lse), _ptr(dq), _ptr(dkc), _ptr(dvc), _ptr(dw),
                                    _ptr(ws), nbytes, _stream(q.device))
         _lib.check(rc, "gca_bwd_indexed")
-        return dq, dkc.to(k_cache.dtype), dvc.to(v_cache.dtype), None, dw.to(ctx.w_dtype), None, None
+        return dq, dkc, dvc, None, dw.to(ctx.w_dtype), None, None
 
 
 def attention_indexed(q, k_cache, v_cache, indices, weights, sm_scale, sm_n=0.0):
