@@ -146,6 +146,9 @@ def main():
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--sm-n", type=float, default=1.0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a 1 GiB device-to-device copy (a kernel of known traffic, for scaling "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (sharding is described in DESIGN.md)")
@@ -169,6 +172,14 @@ def main():
         w = weights[:, :-1].reshape(Z, -1).contiguous().requires_grad_(True)
         o = gca_hip.attention_indexed(q, ck, cv, idx, w, sm_scale, args.sm_n)
         return torch.autograd.grad(o, (q, ck, cv, w), do)
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 29, device=dev, dtype=torch.bfloat16).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()

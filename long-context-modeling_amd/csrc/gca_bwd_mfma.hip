@@ -36,7 +36,7 @@ constexpr int SEG_MAX = 16;   // references per dkdv workgroup in the indexed fo
 // ------------------------------------------------------------------------------------------- dq
 
 template <int D, int GS, bool INDEXED>
-__global__ void __launch_bounds__(128 * GS)
+__global__ void __launch_bounds__(128 * GS) __attribute__((amdgpu_waves_per_eu(D == 64 ? 2 : 1)))
 gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
                        const uint16_t* __restrict__ v, const int64_t* __restrict__ indices,
                        const void* __restrict__ w, int w_is_bf16, const uint16_t* __restrict__ dout,
@@ -195,7 +195,7 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
 // ------------------------------------------------------------------------------------------- dkdv
 
 template <int D, bool INDEXED>
-__global__ void __launch_bounds__(128)
+__global__ void __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(D == 64 ? 2 : 1)))
 gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
                          const uint16_t* __restrict__ v, const void* __restrict__ w, int w_is_bf16,
                          const uint16_t* __restrict__ dout, const float* __restrict__ lse,
