@@ -227,27 +227,33 @@ gca_bwd_dkdv_generic_kernel(Params p, const T* __restrict__ q, const T* __restri
     }
 }
 
-// dw[z, j] = sum_{h, m} delta[z, h, j, m]   (one wavefront per (z, j), fixed summation order)
-__global__ void __launch_bounds__(64)
+// dw[z, j] = sum_{h, m} delta[z, h, j, m].  One workgroup per z: delta[z] is Hq*K rows of Q_CTX
+// contiguous floats; wavefront w sums rows w, w+4, ... (lanes along the row, then a butterfly) into
+// its own per-j partials, which are added in wavefront order -- a fixed summation order.
+constexpr int DW_MAX_K = 256;
+__global__ void __launch_bounds__(256)
 gca_bwd_dw_kernel(Params p, const float* __restrict__ delta, float* __restrict__ dw) {
-    const int64_t zj = blockIdx.x;
-    const int64_t z = zj / p.K;
-    const int j = (int)(zj % p.K);
-    float acc = 0.f;
-    const int total = p.Hq * p.Q_CTX;
-    for (int i = threadIdx.x; i < total; i += 64) {
-        const int h = i / p.Q_CTX, m = i % p.Q_CTX;
-        acc += delta[((z * p.Hq + h) * (int64_t)p.K + j) * p.Q_CTX + m];
-    }
+    __shared__ float part[4][DW_MAX_K];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t z = blockIdx.x;
+    for (int j = lane; j < p.K; j += 64) part[wave][j] = 0.f;
+    const float* dz = delta + z * (int64_t)p.Hq * p.K * p.Q_CTX;
+    const int rows = p.Hq * p.K;
+    for (int r = wave; r < rows; r += 4) {
+        float acc = 0.f;
+        for (int m = lane; m < p.Q_CTX; m += 64) acc += dz[(int64_t)r * p.Q_CTX + m];
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
-    if (threadIdx.x == 0) dw[zj] = acc;
+        for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+        if (lane == 0) part[wave][r % p.K] += acc;
+    }
+    __syncthreads();
+    for (int j = threadIdx.x; j < p.K; j += 256) dw[z * p.K + j] = (part[0][j] + part[1][j]) + (part[2][j] + part[3][j]);
 }
 
 int launch_dw(const Params& p, const float* delta, float* dw, hipStream_t s) {
-    const int64_t blocks = p.Z * p.K;
-    if (blocks <= 0 || blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
-    hipLaunchKernelGGL(gca_bwd_dw_kernel, dim3((unsigned)blocks), dim3(64), 0, s, p, delta, dw);
+    if (p.Z <= 0 || p.Z > 0x7fffffffLL) return GCA_ERR_SHAPE;
+    if (p.K > DW_MAX_K) return GCA_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(gca_bwd_dw_kernel, dim3((unsigned)p.Z), dim3(256), 0, s, p, delta, dw);
     return hipGetLastError() == hipSuccess ? GCA_OK : GCA_ERR_LAUNCH;
 }
 

@@ -4,11 +4,11 @@
 // belongs to sequence n.  The dk/dv kernels are chunk-centric: one workgroup sums the contributions
 // of a chunk's references, so every cache gradient is written exactly once, in a fixed order, with
 // no atomics and no zero-fill.  Lists are built on the device in three launches:
-//   count  per (sequence, block of 256 chunks): the sequence's indices go through LDS, each thread
-//          counts the references of one chunk
+//   count  one wavefront per chunk sweeps the sequence's indices 64 at a time (ballot + popcount)
 //   scan   one workgroup: exclusive scans giving each chunk its list start, its first segment and
 //          its first partial slot
-//   fill   same walk as count; writes the reference ids (ascending per chunk) and the segment table
+//   fill   same walk; a matching lane's rank in the ballot is its place in the list, so the reference
+//          ids come out ascending per chunk; lane 0 writes the chunk's rows of the segment table
 // A chunk's list is cut into segments of at most seg_max references, one dk/dv workgroup each
 // (load balance: popular chunks can be referenced by every later query chunk).  A chunk with one
 // segment (or none: then the segment is empty and the workgroup writes zeros) is stored directly;

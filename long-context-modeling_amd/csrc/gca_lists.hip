@@ -2,8 +2,6 @@
 
 namespace gca {
 
-constexpr int LIST_TILE = 8192;   // references of a sequence held in LDS at a time
-
 int64_t list_seg_bound(const Params& p, int seg_max) { return p.N * p.C + (p.Z * p.K + seg_max - 1) / seg_max; }
 int64_t list_slot_bound(const Params& p, int seg_max) { return 2 * ((p.Z * p.K + seg_max - 1) / seg_max) + 1; }
 
@@ -37,37 +35,31 @@ ListWs list_carve(const Params& p, int seg_max, void* base_v) {
     return ws;
 }
 
-// grid (ceil(C/256), N).  FILL = false: count.  FILL = true: write refs and the segment table.
+// One wavefront per cache chunk: the lanes sweep the sequence's indices 64 at a time; a ballot gives
+// the number of matches and each matching lane's rank, so lists come out ascending without sorting.
+// grid (ceil(C/4), N), 256 threads.  FILL = false: count.  FILL = true: refs and the segment table.
 template <bool FILL>
 __global__ void __launch_bounds__(256)
 gca_list_walk_kernel(Params p, int seg_max, const int64_t* __restrict__ indices, ListWs ws) {
-    __shared__ int s_idx[LIST_TILE];
-    const int tid = threadIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t n = blockIdx.y;
-    const int64_t c = (int64_t)blockIdx.x * 256 + tid;
-    const bool live = c < p.C;
+    const int64_t c = (int64_t)blockIdx.x * 4 + wave;
+    if (c >= p.C) return;
     const int64_t cc = n * p.C + c;
     const int64_t nref = p.zpn * p.K;           // references of this sequence
     const int64_t r0 = n * nref;
     int cnt = 0;
-    const int start = (FILL && live) ? ws.start[cc] : 0;
-    for (int64_t base = 0; base < nref; base += LIST_TILE) {
-        const int m = (int)min((int64_t)LIST_TILE, nref - base);
-        __syncthreads();
-        for (int i = tid; i < m; i += 256) s_idx[i] = (int)clamp_idx(indices[r0 + base + i], p.C);
-        __syncthreads();
-        if (live) {
-            const int ci = (int)c;
-#pragma unroll 8
-            for (int i = 0; i < m; ++i) {
-                if (s_idx[i] == ci) {
-                    if (FILL) ws.refs[start + cnt] = (int)(r0 + base + i);
-                    ++cnt;
-                }
-            }
-        }
+    const int start = FILL ? ws.start[cc] : 0;
+    const unsigned long long below = (1ull << lane) - 1ull;
+#pragma unroll 4
+    for (int64_t base = 0; base < nref; base += 64) {
+        const int64_t i = base + lane;
+        const bool match = i < nref && clamp_idx(indices[r0 + i], p.C) == c;
+        const unsigned long long mask = __ballot(match);
+        if (FILL && match) ws.refs[start + cnt + __popcll(mask & below)] = (int)(r0 + i);
+        cnt += __popcll(mask);
     }
-    if (!live) return;
+    if (lane != 0) return;
     if (!FILL) {
         ws.count[cc] = cnt;
     } else {
@@ -120,7 +112,7 @@ gca_list_scan_kernel(Params p, int seg_max, ListWs ws) {
 
 int list_build(const Params& p, int seg_max, const int64_t* indices, const ListWs& ws, hipStream_t s) {
     if (p.N > 65535) return GCA_ERR_SHAPE;
-    const dim3 grid((unsigned)((p.C + 255) / 256), (unsigned)p.N);
+    const dim3 grid((unsigned)((p.C + 3) / 4), (unsigned)p.N);
     hipLaunchKernelGGL((gca_list_walk_kernel<false>), grid, dim3(256), 0, s, p, seg_max, indices, ws);
     hipLaunchKernelGGL(gca_list_scan_kernel, dim3(1), dim3(1024), 0, s, p, seg_max, ws);
     hipLaunchKernelGGL((gca_list_walk_kernel<true>), grid, dim3(256), 0, s, p, seg_max, indices, ws);

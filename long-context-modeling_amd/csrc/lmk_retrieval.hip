@@ -181,7 +181,8 @@ int launch_lmk_score(const lmk_desc& d, const void* lq, const void* lk, void* sc
 
 // ------------------------------------------------------------------------------------ top-k
 
-constexpr int TOPK_TILE = 2048;      // keys per LDS tile
+constexpr int TOPK_TILE = 2048;      // keys per LDS tile (rows longer than TOPK_SMALL)
+constexpr int TOPK_SMALL = 256;      // tile for short rows: fewer sorting stages
 constexpr int TOPK_THREADS = 256;
 constexpr int TOPK_MAX_KP = 128;     // largest supported power-of-two k
 
@@ -200,14 +201,15 @@ __device__ __forceinline__ void cmpx(uint64_t* keys, int lo, int hi, bool desc) 
     if ((a < b) == desc) { keys[lo] = b; keys[hi] = a; }
 }
 
-// Leaves the kp largest of keys[0, TOPK_TILE) in keys[0, kp), sorted descending.
+// Leaves the kp largest of keys[0, TILE) in keys[0, kp), sorted descending.
 // kp is a power of two <= TOPK_MAX_KP.  All TOPK_THREADS threads of the workgroup must call it.
+template <int TILE>
 __device__ void block_topk(uint64_t* keys, int kp, int tid) {
     // sort groups of kp; even groups descending, odd groups ascending
     for (int size = 2; size <= kp; size <<= 1) {
         for (int stride = size >> 1; stride > 0; stride >>= 1) {
             __syncthreads();
-            for (int i = tid; i < TOPK_TILE / 2; i += TOPK_THREADS) {
+            for (int i = tid; i < TILE / 2; i += TOPK_THREADS) {
                 const int lo = (i / stride) * 2 * stride + (i % stride);
                 cmpx(keys, lo, lo + stride, (lo & size) == 0);
             }
@@ -215,9 +217,9 @@ __device__ void block_topk(uint64_t* keys, int kp, int tid) {
     }
     // halve: (descending group, ascending group) is bitonic; the element-wise maximum keeps the
     // kp largest as a bitonic sequence, which one merge pass sorts again
-    for (int n = TOPK_TILE; n > kp; n >>= 1) {
+    for (int n = TILE; n > kp; n >>= 1) {
         __syncthreads();
-        constexpr int PER = TOPK_TILE / 2 / TOPK_THREADS;
+        constexpr int PER = (TILE / 2 + TOPK_THREADS - 1) / TOPK_THREADS;
         uint64_t tmp[PER];
         const int half = n >> 1;
 #pragma unroll
@@ -278,12 +280,12 @@ __device__ void emit_row(const lmk_desc& d, const uint64_t* keys, int kk, int64_
 // grid (nseg, R).  Segment `seg` of row `row` covers candidates [seg*seg_len, (seg+1)*seg_len)
 // clipped to the part of the row that can be selected.  nseg == 1 writes the final result,
 // otherwise the kp winners of the segment go to ws[(row*nseg + seg)*kp ...].
-template <typename T>
+template <typename T, int TILE>
 __global__ void __launch_bounds__(TOPK_THREADS)
 lmk_topk_kernel(lmk_desc d, int kk, int kp, int nseg, int64_t seg_len, int64_t row0, const T* __restrict__ scores,
                 const T* __restrict__ noise, int64_t* __restrict__ indices, float* __restrict__ weights,
                 uint64_t* __restrict__ ws) {
-    __shared__ uint64_t keys[TOPK_TILE];
+    __shared__ uint64_t keys[TILE];
     __shared__ float sval[TOPK_MAX_KP];
     const int tid = threadIdx.x;
     const int seg = blockIdx.x;
@@ -298,7 +300,7 @@ lmk_topk_kernel(lmk_desc d, int kk, int kp, int nseg, int64_t seg_len, int64_t r
     int carry = 0;   // keys[0, carry) hold the running winners
     int64_t pos = lo;
     do {
-        const int64_t take = TOPK_TILE - carry;
+        const int64_t take = TILE - carry;
         for (int i = tid; i < take; i += TOPK_THREADS) {
             const int64_t e = pos + i;
             uint64_t key = 0;
@@ -310,7 +312,7 @@ lmk_topk_kernel(lmk_desc d, int kk, int kp, int nseg, int64_t seg_len, int64_t r
             }
             keys[carry + i] = key;
         }
-        block_topk(keys, kp, tid);
+        block_topk<TILE>(keys, kp, tid);
         carry = kp;
         pos += take;
     } while (pos < hi);
@@ -341,7 +343,7 @@ lmk_topk_merge_kernel(lmk_desc d, int kk, int kp, int nseg, int64_t row0, const 
             const int64_t e = pos + i;
             keys[carry + i] = e < total ? ws[row * total + e] : 0;
         }
-        block_topk(keys, kp, tid);
+        block_topk<TOPK_TILE>(keys, kp, tid);
         carry = kp;
         pos += take;
     } while (pos < total);
@@ -382,9 +384,14 @@ static int launch_topk_t(const lmk_desc& d, const TopkPlan& pl, const void* scor
     const int64_t slab = 65535;
     for (int64_t r0 = 0; r0 < R; r0 += slab) {
         const int64_t rows = (R - r0) < slab ? (R - r0) : slab;
-        hipLaunchKernelGGL((lmk_topk_kernel<T>), dim3((unsigned)pl.nseg, (unsigned)rows), dim3(TOPK_THREADS), 0, s, d,
-                           pl.kk, pl.kp, pl.nseg, pl.seg_len, r0, (const T*)scores, (const T*)noise, indices, weights,
-                           (uint64_t*)ws);
+        if (d.E <= TOPK_SMALL && pl.kp <= TOPK_SMALL / 2)
+            hipLaunchKernelGGL((lmk_topk_kernel<T, TOPK_SMALL>), dim3((unsigned)pl.nseg, (unsigned)rows), dim3(TOPK_THREADS), 0,
+                               s, d, pl.kk, pl.kp, pl.nseg, pl.seg_len, r0, (const T*)scores, (const T*)noise, indices,
+                               weights, (uint64_t*)ws);
+        else
+            hipLaunchKernelGGL((lmk_topk_kernel<T, TOPK_TILE>), dim3((unsigned)pl.nseg, (unsigned)rows), dim3(TOPK_THREADS), 0,
+                               s, d, pl.kk, pl.kp, pl.nseg, pl.seg_len, r0, (const T*)scores, (const T*)noise, indices,
+                               weights, (uint64_t*)ws);
         if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
         if (pl.nseg > 1) {
             hipLaunchKernelGGL((lmk_topk_merge_kernel<T>), dim3((unsigned)rows), dim3(TOPK_THREADS), 0, s, d, pl.kk, pl.kp,
