@@ -53,11 +53,16 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
     const int n = lane & 31, h = lane >> 5;
     const int gs = wave >> 1, qb = wave & 1;
     const int nqt = p.Q_CTX / 64, nslice = p.G / GS;
-    int64_t bid = blockIdx.x;
+    // logical order: (sequence n, kv head, head slice) pair-major, then the pair's rows (z in n, q tile)
+    const int64_t rows = p.zpn * nqt;
+    int64_t bid = xcd_logical(blockIdx.x, p.N * p.Hkv * nslice * rows);
+    if (bid < 0) return;
     const int qt = (int)(bid % nqt); bid /= nqt;
+    const int64_t zin = bid % p.zpn; bid /= p.zpn;
     const int slice = (int)(bid % nslice); bid /= nslice;
     const int hk = (int)(bid % p.Hkv);
-    const int64_t z = bid / p.Hkv;
+    const int64_t nseq = bid / p.Hkv;
+    const int64_t z = nseq * p.zpn + zin;
     const int hq = hk * p.G + slice * GS + gs;
     const int q0 = qt * 64 + qb * 32;
 
@@ -92,8 +97,8 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
     }
     {
         int64_t rs;
-        const uint16_t* kj = chunk_base(p, k, indices, z, hk, 0, rs);
-        const uint16_t* vj = chunk_base(p, v, indices, z, hk, 0, rs);
+        const uint16_t* kj = chunk_base_n(p, k, indices, nseq, z, hk, 0, rs);
+        const uint16_t* vj = chunk_base_n(p, v, indices, nseq, z, hk, 0, rs);
 #pragma unroll
         for (int i = 0; i < LPT; ++i) {
             stage_k[i] = *reinterpret_cast<const u32x4*>(kj + goff[i]);
@@ -116,16 +121,20 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
         const bool more = (j + 1 < p.K);
         if (more) {
             int64_t rs;
-            const uint16_t* kj = chunk_base(p, k, indices, z, hk, j + 1, rs);
-            const uint16_t* vj = chunk_base(p, v, indices, z, hk, j + 1, rs);
+            const uint16_t* kj = chunk_base_n(p, k, indices, nseq, z, hk, j + 1, rs);
+            const uint16_t* vj = chunk_base_n(p, v, indices, nseq, z, hk, j + 1, rs);
 #pragma unroll
             for (int i = 0; i < LPT; ++i) {
                 stage_k[i] = *reinterpret_cast<const u32x4*>(kj + goff[i]);
                 stage_v[i] = *reinterpret_cast<const u32x4*>(vj + goff[i]);
             }
         }
-        const float lse_q = lse[lrow + (int64_t)j * p.Q_CTX];
+        // mult = w_j * sm_scale multiplies dS; it rides in the exponent: Pm = mult * P = exp2(c S - lse + log2 mult).
+        // A slot of weight 0 gives dS = 0: its P is left unscaled (delta is still needed) and the dQ product skipped.
         const float mult = load_w(w, w_is_bf16, z * p.K + j) * p.sm_scale;
+        const bool live = mult > 0.f;
+        const float eoff = lse[lrow + (int64_t)j * p.Q_CTX] - (live ? __builtin_amdgcn_logf(mult) : 0.f);
+        const float dscale = live ? 1.f / mult : 1.f;
         const unsigned char* kb = smem + buf * BUF;
         const unsigned char* vb = kb + TILE;
 
@@ -147,29 +156,32 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float pe = __builtin_amdgcn_exp2f(fmaf(st[t][r], c, -lse_q));
+                const float pe = __builtin_amdgcn_exp2f(fmaf(st[t][r], c, -eoff));
                 st[t][r] = pe;
                 dsum = fmaf(pe, dpt[t][r], dsum);
             }
         dsum += __shfl_xor(dsum, 32);
+        dsum *= dscale;                                   // D_j = rowsum(P * dP)
         if (h == 0) delta[lrow + (int64_t)j * p.Q_CTX] = dsum;
 
-        bf16x8 dsA[4];
+        if (live) {
+            bf16x8 dsA[4];
 #pragma unroll
-        for (int t4 = 0; t4 < 4; ++t4)
+            for (int t4 = 0; t4 < 4; ++t4)
 #pragma unroll
-            for (int s = 0; s < 8; ++s) {
-                const int r = 8 * (t4 & 1) + s;
-                dsA[t4][s] = (__bf16)(st[t4 >> 1][r] * (dpt[t4 >> 1][r] - dsum) * mult);
-            }
+                for (int s = 0; s < 8; ++s) {
+                    const int r = 8 * (t4 & 1) + s;
+                    dsA[t4][s] = (__bf16)(st[t4 >> 1][r] * (dpt[t4 >> 1][r] - dsum));
+                }
 #pragma unroll
-        for (int t4 = 0; t4 < 4; ++t4)
+            for (int t4 = 0; t4 < 4; ++t4)
 #pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                const int o0 = tr.off(t4, db, RB);
-                const bf16x8 b = lds_read_tr_pair(kb + o0, kb + o0 + 8 * RB);
-                dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsA[t4], b, dqacc[db], 0, 0, 0);
-            }
+                for (int db = 0; db < DB; ++db) {
+                    const int o0 = tr.off(t4, db, RB);
+                    const bf16x8 b = lds_read_tr_pair(kb + o0, kb + o0 + 8 * RB);
+                    dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsA[t4], b, dqacc[db], 0, 0, 0);
+                }
+        }
 
         if (more) {
             unsigned char* nb = smem + (buf ^ 1) * BUF;
@@ -341,8 +353,10 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
         }
         const unsigned char* qbuf = smem + buf * BUF;
         const unsigned char* dobuf = qbuf + TILE;
-        const float wj = w_cur, wsj = w_cur * p.sm_scale;
+        // P~ = w P rides in the exponent (exp2(c S - lse + log2 w)); a slot of weight 0 adds nothing to dk, dv
+        const float lw = __builtin_amdgcn_logf(w_cur);
 
+        if (w_cur > 0.f) {
 #pragma unroll
         for (int qt = 0; qt < 2; ++qt) {
             // S = Q K^T, dP = dO V^T for 32 query rows: queries in registers, key n in the lane
@@ -360,14 +374,14 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
                 // registers 4a .. 4a+3 are queries 32*qt + 8a + 4h + 0..3
-                const f32x4 l4 = *reinterpret_cast<const f32x4*>(&s_lse[buf][32 * qt + 8 * a + 4 * h]);
-                const f32x4 d4 = *reinterpret_cast<const f32x4*>(&s_dl[buf][32 * qt + 8 * a + 4 * h]);
+                f32x4 l4 = *reinterpret_cast<const f32x4*>(&s_lse[buf][32 * qt + 8 * a + 4 * h]);
+                f32x4 d4 = *reinterpret_cast<const f32x4*>(&s_dl[buf][32 * qt + 8 * a + 4 * h]);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int r = 4 * a + e;
-                    const float pe = __builtin_amdgcn_exp2f(fmaf(s[r], c, -l4[e]));
-                    pA[r >> 3][r & 7] = (__bf16)(pe * wj);
-                    dsA[r >> 3][r & 7] = (__bf16)(pe * (dp[r] - d4[e]) * wsj);
+                    const float pw = __builtin_amdgcn_exp2f(fmaf(s[r], c, lw - l4[e]));
+                    pA[r >> 3][r & 7] = (__bf16)pw;
+                    dsA[r >> 3][r & 7] = (__bf16)(pw * fmaf(dp[r], p.sm_scale, -d4[e] * p.sm_scale));
                 }
             }
             // dV += P~^T dO, dK += dS^T Q over these 32 queries (two 16-query reduction steps)
@@ -384,6 +398,7 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
                 }
             }
         }
+        }
 
         if (more) {
             unsigned char* nb = smem + (buf ^ 1) * BUF;
@@ -399,21 +414,28 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
     }
 
     // ---- write the tile: register r of block db is key row 32*kbw + 8*(r/4) + 4*h + r%4, column 32*db + n
+    if (INDEXED && slot >= 0) {
+        float* part = ws.partials + ((int64_t)slot * p.Hkv + hk) * 2 * (64 * D) + 32 * kbw * D + n;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+        for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int row = 32 * kbw + 8 * (r >> 2) + 4 * h + (r & 3);
-            const int64_t off = out_off + (int64_t)row * rs + 32 * db + n;
-            if (INDEXED && slot >= 0) {
-                float* part = ws.partials + ((int64_t)slot * p.Hkv + hk) * 2 * (64 * D) + row * D + 32 * db + n;
-                part[0] = dkacc[db][r];
-                part[64 * D] = dvacc[db][r];
-            } else {
-                ((uint16_t*)dk_out)[off] = bf16_bits(dkacc[db][r]);
-                ((uint16_t*)dv_out)[off] = bf16_bits(dvacc[db][r]);
+            for (int r = 0; r < 16; ++r) {
+                const int row = 8 * (r >> 2) + 4 * h + (r & 3);
+                part[row * D + 32 * db] = dkacc[db][r];
+                part[64 * D + row * D + 32 * db] = dvacc[db][r];
             }
-        }
+    } else {
+        uint16_t* dkp = (uint16_t*)dk_out + out_off + (int64_t)(32 * kbw) * rs + n;
+        uint16_t* dvp = (uint16_t*)dv_out + out_off + (int64_t)(32 * kbw) * rs + n;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = 8 * (r >> 2) + 4 * h + (r & 3);
+                dkp[row * rs + 32 * db] = bf16_bits(dkacc[db][r]);
+                dvp[row * rs + 32 * db] = bf16_bits(dvacc[db][r]);
+            }
+    }
 }
 
 // Chunks whose list was cut into several segments: add the float partial tiles in segment order.
@@ -446,7 +468,7 @@ gca_bwd_dkdv_reduce_kernel(Params p, int seg_max, uint16_t* __restrict__ dk_out,
 template <int D, int GS>
 static int launch_dq_gs(const Params& p, const void* q, const void* k, const void* v, const int64_t* idx, const void* w,
                         int wb, const void* dout, const float* lse, void* dq, float* delta, hipStream_t s) {
-    const int64_t blocks = p.Z * p.Hkv * (p.G / GS) * (p.Q_CTX / 64);
+    const int64_t blocks = xcd_grid(p.Z * p.Hkv * (p.G / GS) * (p.Q_CTX / 64));
     if (blocks <= 0 || blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
     if (p.indexed)
         hipLaunchKernelGGL((gca_bwd_dq_mfma_kernel<D, GS, true>), dim3((unsigned)blocks), dim3(128 * GS), 0, s, p,

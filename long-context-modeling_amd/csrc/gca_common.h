@@ -56,10 +56,9 @@ inline Params make_params(const gca_desc& d, bool indexed) {
 // distance in elements between consecutive key rows.  Gathered form: k is (Z,Hkv,K,K_CTX,D);
 // indexed form: cache is (N,C,K_CTX,Hkv*D) and the chunk id comes from indices[z,j].
 template <typename T>
-__device__ __forceinline__ const T* chunk_base(const Params& p, const T* base, const int64_t* indices,
-                                               int64_t z, int hk, int j, int64_t& row_stride) {
+__device__ __forceinline__ const T* chunk_base_n(const Params& p, const T* base, const int64_t* indices,
+                                                 int64_t n, int64_t z, int hk, int j, int64_t& row_stride) {
     if (p.indexed) {
-        const int64_t n = z / p.zpn;
         int64_t c = indices[z * p.K + j];
         c = c < 0 ? 0 : (c >= p.C ? p.C - 1 : c);   // out-of-range ids never leave the cache
         row_stride = (int64_t)p.Hkv * p.D;
@@ -67,6 +66,13 @@ __device__ __forceinline__ const T* chunk_base(const Params& p, const T* base, c
     }
     row_stride = p.D;
     return base + (((z * p.Hkv + hk) * p.K + j) * (int64_t)p.K_CTX) * p.D;
+}
+
+// Same, for callers that do not know the row's sequence n = z / zpn yet.
+template <typename T>
+__device__ __forceinline__ const T* chunk_base(const Params& p, const T* base, const int64_t* indices,
+                                               int64_t z, int hk, int j, int64_t& row_stride) {
+    return chunk_base_n(p, base, indices, p.indexed ? z / p.zpn : 0, z, hk, j, row_stride);
 }
 
 }  // namespace gca

@@ -33,7 +33,7 @@ template <int D> struct FwdCfg {
 };
 
 template <int D, int GS, bool INDEXED>
-__global__ void __launch_bounds__(128 * GS)
+__global__ void __launch_bounds__(128 * GS) __attribute__((amdgpu_waves_per_eu(2)))
 gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
                     const uint16_t* __restrict__ v, const int64_t* __restrict__ indices,
                     const void* __restrict__ w, int w_is_bf16, uint16_t* __restrict__ o, float* __restrict__ lse) {
@@ -52,14 +52,18 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
     const int n = lane & 31, h = lane >> 5;
     const int gs = wave >> 1, qb = wave & 1;
 
-    // block -> (z, hk, slice, qt); consecutive blocks share z so that they touch neighbouring memory
     const int nqt = p.Q_CTX / 64;
     const int nslice = p.G / GS;
-    int64_t bid = blockIdx.x;
+    // logical order: (sequence n, kv head, head slice) pair-major, then the pair's rows (z in n, q tile)
+    const int64_t rows = p.zpn * nqt;
+    int64_t bid = xcd_logical(blockIdx.x, p.N * p.Hkv * nslice * rows);
+    if (bid < 0) return;
     const int qt = (int)(bid % nqt); bid /= nqt;
+    const int64_t zin = bid % p.zpn; bid /= p.zpn;
     const int slice = (int)(bid % nslice); bid /= nslice;
     const int hk = (int)(bid % p.Hkv);
-    const int64_t z = bid / p.Hkv;
+    const int64_t nseq = bid / p.Hkv;
+    const int64_t z = nseq * p.zpn + zin;
     const int hq = hk * p.G + slice * GS + gs;
     const int q0 = qt * 64 + qb * 32;
 
@@ -96,8 +100,8 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
     }
     {
         int64_t rs;
-        const uint16_t* kj = chunk_base(p, k, indices, z, hk, 0, rs);
-        const uint16_t* vj = chunk_base(p, v, indices, z, hk, 0, rs);
+        const uint16_t* kj = chunk_base_n(p, k, indices, nseq, z, hk, 0, rs);
+        const uint16_t* vj = chunk_base_n(p, v, indices, nseq, z, hk, 0, rs);
 #pragma unroll
         for (int i = 0; i < LPT; ++i) {
             stage_k[i] = *reinterpret_cast<const u32x4*>(kj + goff[i]);
@@ -119,8 +123,8 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
         const bool more = (j + 1 < p.K);
         if (more) {
             int64_t rs;
-            const uint16_t* kj = chunk_base(p, k, indices, z, hk, j + 1, rs);
-            const uint16_t* vj = chunk_base(p, v, indices, z, hk, j + 1, rs);
+            const uint16_t* kj = chunk_base_n(p, k, indices, nseq, z, hk, j + 1, rs);
+            const uint16_t* vj = chunk_base_n(p, v, indices, nseq, z, hk, j + 1, rs);
 #pragma unroll
             for (int i = 0; i < LPT; ++i) {
                 stage_k[i] = *reinterpret_cast<const u32x4*>(kj + goff[i]);
@@ -219,7 +223,7 @@ bool mfma_supported(const gca_desc& d) {
 template <int D, int GS>
 static int launch_gs(const Params& p, const void* q, const void* k, const void* v, const int64_t* idx,
                      const void* w, int w_is_bf16, void* o, float* lse, hipStream_t s) {
-    const int64_t blocks = p.Z * p.Hkv * (p.G / GS) * (p.Q_CTX / 64);
+    const int64_t blocks = xcd_grid(p.Z * p.Hkv * (p.G / GS) * (p.Q_CTX / 64));
     if (blocks <= 0 || blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
     if (p.indexed)
         hipLaunchKernelGGL((gca_fwd_mfma_kernel<D, GS, true>), dim3((unsigned)blocks), dim3(128 * GS), 0, s, p,

@@ -63,6 +63,19 @@ struct TrLane {
     }
 };
 
+// XCD-aware work order.  The hardware deals workgroups round-robin to the 8 XCDs (workgroup i runs
+// on XCD i % 8), each with its own L2.  Work items are numbered so that items sharing data are
+// consecutive ("logical" order); XCD x takes the contiguous range [x*per, (x+1)*per) of it, so the
+// tiles one (sequence, head) pair re-reads stay in one L2.  Launch 8*per workgroups, per = ceil(T/8);
+// returns -1 for the padding workgroups.
+constexpr int NUM_XCD = 8;
+__device__ __forceinline__ int64_t xcd_logical(int64_t bid, int64_t total) {
+    const int64_t per = (total + NUM_XCD - 1) / NUM_XCD;
+    const int64_t logical = (bid % NUM_XCD) * per + bid / NUM_XCD;
+    return logical < total ? logical : -1;
+}
+inline int64_t xcd_grid(int64_t total) { return (total + NUM_XCD - 1) / NUM_XCD * NUM_XCD; }
+
 __device__ __forceinline__ float load_w(const void* w, int w_is_bf16, int64_t i) {
     return w_is_bf16 ? bf16_bits_to_f(((const uint16_t*)w)[i]) : ((const float*)w)[i];
 }
