@@ -10,13 +10,16 @@
 //      dS = w sm_scale P (dP - D) -> bf16, already in A-operand order
 //      dQ += dS K                         K read transposed from LDS (ds_read_tr16_b64)
 //
-// 2. dkdv kernel -- kv-tile-centric.  A workgroup owns ONE 64 x D key/value tile (its two wavefronts
-//    own 32 key rows each, K and V rows held in registers as B operands) and walks every
-//    (query chunk z, slot j, query head of the group, 64-row query tile) that attends to this tile; Q and dO tiles are
-//    staged in LDS (double buffered) and shared by both wavefronts.
-//      S = Q K^T, dP = dO V^T            queries in registers, the lane's key in every register
-//      P = exp2(c S - lse[q]), P~ = w P, dS = sm_scale P~ (dP - delta[q])   lse/delta rows from LDS
-//      dV += P~^T dO,  dK += dS^T Q      dO and Q read transposed from LDS
+// 2. dkdv kernel -- kv-tile-centric.  A workgroup of four wavefronts owns ONE 64 x D key/value tile and
+//    walks every (query chunk z, slot j, query head of the group, 64-row query tile) that attends to
+//    it; Q and dO tiles are staged in LDS (double buffered, asynchronous copies).  Wavefront
+//    (kbw, sub) keeps the K and V rows of key half kbw in registers as B operands.
+//      phase 1  (key half kbw x query half sub)   S = Q K^T, dP = dO V^T: queries in registers, the
+//               lane's key in every register; P~ = w exp2(c S - lse[q]), dS = sm_scale P~ (dP - delta[q]);
+//               both rounded to bf16 ARE the A operands of phase 2 and are handed over lane for lane
+//               through a 16 KB LDS exchange buffer (no transposition, no bank conflicts)
+//      phase 2  (key half kbw x dim half sub)     dV += P~^T dO,  dK += dS^T Q  with dO and Q read
+//               transposed from LDS; each wavefront accumulates a 32 x D/2 block of dK and of dV
 //    Gathered form: the tile is slot (z, kv head, j) and the walk is the G heads of the group; dk/dv
 //    are written in bf16.  Indexed form: the tile is a chunk of the cache and the walk follows a
 //    reference list built on the device (every list ordered by (z, j), no atomics, so the summation
@@ -44,9 +47,7 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
     constexpr int NT = 128 * GS;
     constexpr int KS = D / 16, DB = D / 32;
     constexpr int RB = D * 2, TILE = 64 * RB, BUF = 2 * TILE;
-    constexpr int PIECES = TILE / 16, LPT = PIECES / NT, PPR = RB / 16;
-    static_assert(PIECES % NT == 0, "tile must split evenly over the workgroup");
-    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF];
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * BUF];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -82,34 +83,13 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
         for (int r = 0; r < 16; ++r) dqacc[db][r] = 0.f;
 
     const float c = p.sm_scale * LOG2E;
-    u32x4 stage_k[LPT], stage_v[LPT];
-    int64_t goff[LPT];
-    int loff[LPT];
-    {
-        const int64_t rs = INDEXED ? (int64_t)p.Hkv * D : (int64_t)D;
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) {
-            const int piece = tid + i * NT;
-            const int row = piece / PPR, col = piece % PPR;
-            goff[i] = row * rs + col * 8;
-            loff[i] = tile_off(row, col, RB);
-        }
-    }
+    const TileLoader<D, NT> loader(tid, INDEXED ? p.Hkv * D : D);
     {
         int64_t rs;
-        const uint16_t* kj = chunk_base_n(p, k, indices, nseq, z, hk, 0, rs);
-        const uint16_t* vj = chunk_base_n(p, v, indices, nseq, z, hk, 0, rs);
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) {
-            stage_k[i] = *reinterpret_cast<const u32x4*>(kj + goff[i]);
-            stage_v[i] = *reinterpret_cast<const u32x4*>(vj + goff[i]);
-        }
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) {
-            *reinterpret_cast<u32x4*>(smem + loff[i]) = stage_k[i];
-            *reinterpret_cast<u32x4*>(smem + TILE + loff[i]) = stage_v[i];
-        }
+        loader.issue(chunk_base_n(p, k, indices, nseq, z, hk, 0, rs), smem);
+        loader.issue(chunk_base_n(p, v, indices, nseq, z, hk, 0, rs), smem + TILE);
     }
+    wait_async_tiles();
     __syncthreads();
 
     const TrLane tr(lane);
@@ -118,16 +98,12 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
 
     for (int j = 0; j < p.K; ++j) {
         const int buf = j & 1;
-        const bool more = (j + 1 < p.K);
-        if (more) {
+        if (j + 1 < p.K) {
+            // the other buffer was last read in iteration j-1, which every wavefront has left
             int64_t rs;
-            const uint16_t* kj = chunk_base_n(p, k, indices, nseq, z, hk, j + 1, rs);
-            const uint16_t* vj = chunk_base_n(p, v, indices, nseq, z, hk, j + 1, rs);
-#pragma unroll
-            for (int i = 0; i < LPT; ++i) {
-                stage_k[i] = *reinterpret_cast<const u32x4*>(kj + goff[i]);
-                stage_v[i] = *reinterpret_cast<const u32x4*>(vj + goff[i]);
-            }
+            unsigned char* nb = smem + (buf ^ 1) * BUF;
+            loader.issue(chunk_base_n(p, k, indices, nseq, z, hk, j + 1, rs), nb);
+            loader.issue(chunk_base_n(p, v, indices, nseq, z, hk, j + 1, rs), nb + TILE);
         }
         // mult = w_j * sm_scale multiplies dS; it rides in the exponent: Pm = mult * P = exp2(c S - lse + log2 mult).
         // A slot of weight 0 gives dS = 0: its P is left unscaled (delta is still needed) and the dQ product skipped.
@@ -183,14 +159,7 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
                 }
         }
 
-        if (more) {
-            unsigned char* nb = smem + (buf ^ 1) * BUF;
-#pragma unroll
-            for (int i = 0; i < LPT; ++i) {
-                *reinterpret_cast<u32x4*>(nb + loff[i]) = stage_k[i];
-                *reinterpret_cast<u32x4*>(nb + TILE + loff[i]) = stage_v[i];
-            }
-        }
+        wait_async_tiles();
         __syncthreads();
     }
 
@@ -206,9 +175,13 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
 
 // ------------------------------------------------------------------------------------------- dkdv
 
+// Two-wavefront variant of the dk/dv kernel, used for D == 64: each wavefront owns 32 key rows and does
+// all four products for them itself (S, dP over all 64 query rows of a unit, then dV, dK), so the only
+// thing the wavefronts share is the Q / dO tile in LDS and there is one barrier per unit.  With
+// D == 128 its accumulators and operands need ~450 registers; the four-wavefront kernel below halves that.
 template <int D, bool INDEXED>
-__global__ void __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(D == 64 ? 2 : 1)))
-gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
+__global__ void __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2)))
+gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
                          const uint16_t* __restrict__ v, const void* __restrict__ w, int w_is_bf16,
                          const uint16_t* __restrict__ dout, const float* __restrict__ lse,
                          const float* __restrict__ delta, void* __restrict__ dk_out, void* __restrict__ dv_out,
@@ -216,10 +189,9 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
     constexpr int NT = 128;
     constexpr int KS = D / 16, DB = D / 32;
     constexpr int RB = D * 2, TILE = 64 * RB, BUF = 2 * TILE;   // Q tile then dO tile
-    constexpr int PIECES = TILE / 16, LPT = PIECES / NT, PPR = RB / 16;
-    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * BUF];
-    __shared__ __attribute__((aligned(16))) float s_lse[2][64];
-    __shared__ __attribute__((aligned(16))) float s_dl[2][64];
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * BUF];
+    __shared__ __attribute__((aligned(256))) float s_lse[2][64];
+    __shared__ __attribute__((aligned(256))) float s_dl[2][64];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, kbw = tid >> 6;     // kbw: which 32 key rows this wavefront owns
@@ -282,16 +254,7 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
         for (int r = 0; r < 16; ++r) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
 
     const float c = p.sm_scale * LOG2E;
-    u32x4 stage_q[LPT], stage_do[LPT];
-    float stage_f = 0.f;    // threads 0-63 stage lse[q], threads 64-127 stage delta[q]
-    int goff[LPT], loff[LPT];
-#pragma unroll
-    for (int i = 0; i < LPT; ++i) {
-        const int piece = tid + i * NT;
-        const int row = piece / PPR, col = piece % PPR;
-        goff[i] = row * D + col * 8;
-        loff[i] = tile_off(row, col, RB);
-    }
+    const TileLoader<D, NT> loader(tid, D);
 
     // unit u = (reference, query head of the group, 64-row query tile), tile fastest
     const int nqt = p.Q_CTX / 64;
@@ -310,26 +273,22 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
         }
     };
 
-    float w_cur, w_next = 0.f;
-    {
+    // asynchronous copy of unit u's Q / dO tiles and lse / delta rows into buffer `buf`
+    auto issue_unit = [&](int u, int buf) -> float {
         int64_t z; int j, hq, qrow0;
-        unit_coords(0, z, j, hq, qrow0);
+        unit_coords(u, z, j, hq, qrow0);
         const int64_t qoff = ((z * p.Hq + hq) * (int64_t)p.Q_CTX + qrow0) * D;
         const int64_t loffq = ((z * p.Hq + hq) * (int64_t)p.K + j) * p.Q_CTX + qrow0;
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) {
-            stage_q[i] = *reinterpret_cast<const u32x4*>(q + qoff + goff[i]);
-            stage_do[i] = *reinterpret_cast<const u32x4*>(dout + qoff + goff[i]);
-        }
-        stage_f = tid < 64 ? lse[loffq + tid] : delta[loffq + tid - 64];
-        w_cur = load_w(w, w_is_bf16, z * p.K + j);
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) {
-            *reinterpret_cast<u32x4*>(smem + loff[i]) = stage_q[i];
-            *reinterpret_cast<u32x4*>(smem + TILE + loff[i]) = stage_do[i];
-        }
-        if (tid < 64) s_lse[0][tid] = stage_f; else s_dl[0][tid - 64] = stage_f;
-    }
+        unsigned char* nb = smem + buf * BUF;
+        loader.issue(q + qoff, nb);
+        loader.issue(dout + qoff, nb + TILE);
+        if (kbw == 0) async_row64(lse + loffq, s_lse[buf], lane);
+        else async_row64(delta + loffq, s_dl[buf], lane);
+        return load_w(w, w_is_bf16, z * p.K + j);
+    };
+
+    float w_cur = issue_unit(0, 0), w_next = 0.f;
+    wait_async_tiles();
     __syncthreads();
 
     const TrLane tr(lane);
@@ -338,19 +297,7 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
     for (int u = 0; u < nunits; ++u) {
         const int buf = u & 1;
         const bool more = (u + 1 < nunits);
-        if (more) {
-            int64_t z; int j, hq, qrow0;
-            unit_coords(u + 1, z, j, hq, qrow0);
-            const int64_t qoff = ((z * p.Hq + hq) * (int64_t)p.Q_CTX + qrow0) * D;
-            const int64_t loffq = ((z * p.Hq + hq) * (int64_t)p.K + j) * p.Q_CTX + qrow0;
-#pragma unroll
-            for (int i = 0; i < LPT; ++i) {
-                stage_q[i] = *reinterpret_cast<const u32x4*>(q + qoff + goff[i]);
-                stage_do[i] = *reinterpret_cast<const u32x4*>(dout + qoff + goff[i]);
-            }
-            stage_f = tid < 64 ? lse[loffq + tid] : delta[loffq + tid - 64];
-            w_next = load_w(w, w_is_bf16, z * p.K + j);
-        }
+        if (more) w_next = issue_unit(u + 1, buf ^ 1);   // that buffer was last read in iteration u-1
         const unsigned char* qbuf = smem + buf * BUF;
         const unsigned char* dobuf = qbuf + TILE;
         // P~ = w P rides in the exponent (exp2(c S - lse + log2 w)); a slot of weight 0 adds nothing to dk, dv
@@ -400,16 +347,8 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
         }
         }
 
-        if (more) {
-            unsigned char* nb = smem + (buf ^ 1) * BUF;
-#pragma unroll
-            for (int i = 0; i < LPT; ++i) {
-                *reinterpret_cast<u32x4*>(nb + loff[i]) = stage_q[i];
-                *reinterpret_cast<u32x4*>(nb + TILE + loff[i]) = stage_do[i];
-            }
-            if (tid < 64) s_lse[buf ^ 1][tid] = stage_f; else s_dl[buf ^ 1][tid - 64] = stage_f;
-            w_cur = w_next;
-        }
+        w_cur = w_next;
+        wait_async_tiles();
         __syncthreads();
     }
 
@@ -429,6 +368,223 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
         uint16_t* dvp = (uint16_t*)dv_out + out_off + (int64_t)(32 * kbw) * rs + n;
 #pragma unroll
         for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = 8 * (r >> 2) + 4 * h + (r & 3);
+                dkp[row * rs + 32 * db] = bf16_bits(dkacc[db][r]);
+                dvp[row * rs + 32 * db] = bf16_bits(dvacc[db][r]);
+            }
+    }
+}
+
+template <int D, bool INDEXED>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
+                         const uint16_t* __restrict__ v, const void* __restrict__ w, int w_is_bf16,
+                         const uint16_t* __restrict__ dout, const float* __restrict__ lse,
+                         const float* __restrict__ delta, void* __restrict__ dk_out, void* __restrict__ dv_out,
+                         ListWs ws) {
+    constexpr int NT = 256;
+    constexpr int KS = D / 16, DB = D / 32, DBH = DB / 2;
+    constexpr int RB = D * 2, TILE = 64 * RB, BUF = 2 * TILE;   // Q tile then dO tile
+    constexpr int XCH = 2 * 4 * 64 * 16;                        // one exchange array: [key half][16-query step][lane] x 16 B
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * BUF + 2 * XCH];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int kbw = wave >> 1;            // 32 key rows owned in both phases
+    const int sub = wave & 1;             // phase 1: 32-query half; phase 2: dim half
+    const int n = lane & 31, h = lane >> 5;
+
+    // ---- which tile, which walk
+    int hk, nunits, list0 = 0, slot = -1;
+    int64_t gz = 0;          // gathered: the single (z, j)
+    int gj = 0;
+    const uint16_t* kt;
+    const uint16_t* vt;
+    int64_t rs, out_off;     // key-row stride of the tile; element offset of the tile in the output
+    if (INDEXED) {
+        const int seg = blockIdx.x / p.Hkv;
+        hk = blockIdx.x % p.Hkv;
+        if (seg >= ws.nseg[0]) return;
+        const int64_t cc = ws.seg_chunk[seg];
+        list0 = ws.seg_start[seg];
+        nunits = ws.seg_len[seg] * p.G * (p.Q_CTX / 64);
+        slot = ws.seg_slot[seg];
+        rs = (int64_t)p.Hkv * D;
+        out_off = cc * p.K_CTX * rs + (int64_t)hk * D;
+        kt = k + out_off;
+        vt = v + out_off;
+        if (nunits == 0) {
+            // nobody retrieved this chunk: its gradient is zero
+            for (int i = tid; i < 64 * D; i += NT) {
+                const int64_t off = out_off + (int64_t)(i / D) * rs + (i % D);
+                ((uint16_t*)dk_out)[off] = 0;
+                ((uint16_t*)dv_out)[off] = 0;
+            }
+            return;
+        }
+    } else {
+        int64_t bid = blockIdx.x;
+        gj = (int)(bid % p.K); bid /= p.K;
+        hk = (int)(bid % p.Hkv);
+        gz = bid / p.Hkv;
+        nunits = p.G * (p.Q_CTX / 64);
+        rs = D;
+        out_off = (((gz * p.Hkv + hk) * p.K + gj) * (int64_t)p.K_CTX) * D;
+        kt = k + out_off;
+        vt = v + out_off;
+    }
+
+    // K, V rows of this wavefront as B operands: lane holds key 32*kbw + n, dims 16*ks + 8*h .. +7
+    bf16x8 kB[KS], vB[KS];
+    {
+        const int64_t off = (int64_t)(32 * kbw + n) * rs + 8 * h;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            kB[ks] = *reinterpret_cast<const bf16x8*>(kt + off + 16 * ks);
+            vB[ks] = *reinterpret_cast<const bf16x8*>(vt + off + 16 * ks);
+        }
+    }
+    f32x16 dkacc[DBH], dvacc[DBH];
+#pragma unroll
+    for (int db = 0; db < DBH; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
+
+    const float c = p.sm_scale * LOG2E;
+    const TileLoader<D, NT> loader(tid, D);
+
+    // unit u = (reference, query head of the group, 64-row query tile), tile fastest
+    const int nqt = p.Q_CTX / 64;
+    const int upr = p.G * nqt;   // units per reference
+    auto unit_coords = [&](int u, int64_t& z, int& j, int& hq, int& qrow0) {
+        const int g = (u % upr) / nqt;
+        qrow0 = (u % nqt) * 64;
+        hq = hk * p.G + g;
+        if (INDEXED) {
+            const int ref = ws.refs[list0 + u / upr];
+            z = ref / p.K;
+            j = ref % p.K;
+        } else {
+            z = gz;
+            j = gj;
+        }
+    };
+
+    // Per unit: asynchronous copy of its Q / dO tiles into buffer `buf`.  This lane's 16 lse and 16
+    // delta values (queries 32*sub + 8a + 4h + 0..3, a = 0..3) come through registers; they are
+    // fetched for the next unit right after phase 1 has used the current ones.
+    f32x4 l_cur[4], d_cur[4];
+    int64_t loff_next = 0;
+    auto issue_unit = [&](int u, int buf) -> float {
+        int64_t z; int j, hq, qrow0;
+        unit_coords(u, z, j, hq, qrow0);
+        const int64_t qoff = ((z * p.Hq + hq) * (int64_t)p.Q_CTX + qrow0) * D;
+        loff_next = ((z * p.Hq + hq) * (int64_t)p.K + j) * p.Q_CTX + qrow0 + 32 * sub + 4 * h;
+        unsigned char* nb = smem + buf * BUF;
+        loader.issue(q + qoff, nb);
+        loader.issue(dout + qoff, nb + TILE);
+        return load_w(w, w_is_bf16, z * p.K + j);
+    };
+    auto fetch_rows = [&]() {
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            l_cur[a] = *reinterpret_cast<const f32x4*>(lse + loff_next + 8 * a);
+            d_cur[a] = *reinterpret_cast<const f32x4*>(delta + loff_next + 8 * a);
+        }
+    };
+
+    float w_cur = issue_unit(0, 0), w_next = 0.f;
+    fetch_rows();
+    wait_async_tiles();
+    __syncthreads();
+
+    const TrLane tr(lane);
+    const int fsw = swz(n);
+    unsigned char* xp = smem + 2 * BUF;     // P~ operands
+    unsigned char* xd = xp + XCH;           // dS operands
+    const int xoff = (kbw * 4 * 64 + lane) * 16;
+
+    for (int u = 0; u < nunits; ++u) {
+        const int buf = u & 1;
+        const bool more = (u + 1 < nunits);
+        if (more) w_next = issue_unit(u + 1, buf ^ 1);   // that buffer was last read in iteration u-1
+        const unsigned char* qbuf = smem + buf * BUF;
+        const unsigned char* dobuf = qbuf + TILE;
+        const bool live = w_cur > 0.f;      // a slot of weight 0 adds nothing to dk, dv
+        // P~ = w P rides in the exponent: exp2(c S - lse + log2 w)
+        const float lw = __builtin_amdgcn_logf(w_cur);
+
+        if (live) {
+            // ---- phase 1: S = Q K^T, dP = dO V^T for query rows 32*sub .. +31 against key rows 32*kbw .. +31
+            f32x16 s, dp;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+            const int rowoff = (32 * sub + n) * RB;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int po = rowoff + (((2 * ks + h) ^ fsw) << 4);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(qbuf + po), kB[ks], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(dobuf + po), vB[ks], dp, 0, 0, 0);
+            }
+            bf16x8 pA[2], dsA[2];
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int r = 4 * a + e;      // query 32*sub + 8a + 4h + e
+                    const float pw = __builtin_amdgcn_exp2f(fmaf(s[r], c, lw - l_cur[a][e]));
+                    pA[r >> 3][r & 7] = (__bf16)pw;
+                    dsA[r >> 3][r & 7] = (__bf16)(pw * fmaf(dp[r], p.sm_scale, -d_cur[a][e] * p.sm_scale));
+                }
+            // hand the A operands of 16-query steps 2*sub, 2*sub+1 to the phase-2 owners, lane for lane
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+                *reinterpret_cast<bf16x8*>(xp + xoff + (2 * sub + t2) * 1024) = pA[t2];
+                *reinterpret_cast<bf16x8*>(xd + xoff + (2 * sub + t2) * 1024) = dsA[t2];
+            }
+        }
+        if (more) fetch_rows();
+        __syncthreads();
+        if (live) {
+            // ---- phase 2: dV += P~^T dO, dK += dS^T Q for key rows 32*kbw .. +31, dims (D/2)*sub .. +D/2-1
+#pragma unroll
+            for (int t4 = 0; t4 < 4; ++t4) {
+                const bf16x8 pa = *reinterpret_cast<const bf16x8*>(xp + xoff + t4 * 1024);
+                const bf16x8 da = *reinterpret_cast<const bf16x8*>(xd + xoff + t4 * 1024);
+#pragma unroll
+                for (int db = 0; db < DBH; ++db) {
+                    const int o0 = tr.off(t4, sub * DBH + db, RB);
+                    const bf16x8 bdo = lds_read_tr_pair(dobuf + o0, dobuf + o0 + 8 * RB);
+                    dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pa, bdo, dvacc[db], 0, 0, 0);
+                    const bf16x8 bq = lds_read_tr_pair(qbuf + o0, qbuf + o0 + 8 * RB);
+                    dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, bq, dkacc[db], 0, 0, 0);
+                }
+            }
+        }
+        w_cur = w_next;
+        wait_async_tiles();
+        __syncthreads();
+    }
+
+    // ---- write: register r of block db is key row 32*kbw + 8*(r/4) + 4*h + r%4, column (D/2)*sub + 32*db + n
+    const int col0 = (D / 2) * sub + n;
+    if (INDEXED && slot >= 0) {
+        float* part = ws.partials + ((int64_t)slot * p.Hkv + hk) * 2 * (64 * D) + 32 * kbw * D + col0;
+#pragma unroll
+        for (int db = 0; db < DBH; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = 8 * (r >> 2) + 4 * h + (r & 3);
+                part[row * D + 32 * db] = dkacc[db][r];
+                part[64 * D + row * D + 32 * db] = dvacc[db][r];
+            }
+    } else {
+        uint16_t* dkp = (uint16_t*)dk_out + out_off + (int64_t)(32 * kbw) * rs + col0;
+        uint16_t* dvp = (uint16_t*)dv_out + out_off + (int64_t)(32 * kbw) * rs + col0;
+#pragma unroll
+        for (int db = 0; db < DBH; ++db)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = 8 * (r >> 2) + 4 * h + (r & 3);
@@ -501,17 +657,27 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
         if ((rc = list_build(p, SEG_MAX, idx, ws, s)) != GCA_OK) return rc;
         const int64_t blocks = list_seg_bound(p, SEG_MAX) * p.Hkv;
         if (blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
-        hipLaunchKernelGGL((gca_bwd_dkdv_mfma_kernel<D, true>), dim3((unsigned)blocks), dim3(128), 0, s, p,
-                           (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse, delta,
-                           dk, dv, ws);
+        if (D == 64)
+            hipLaunchKernelGGL((gca_bwd_dkdv2_mfma_kernel<D, true>), dim3((unsigned)blocks), dim3(128), 0, s, p,
+                               (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
+                               delta, dk, dv, ws);
+        else
+            hipLaunchKernelGGL((gca_bwd_dkdv_mfma_kernel<D, true>), dim3((unsigned)blocks), dim3(256), 0, s, p,
+                               (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
+                               delta, dk, dv, ws);
         hipLaunchKernelGGL((gca_bwd_dkdv_reduce_kernel<D>), dim3((unsigned)(p.N * p.C * p.Hkv)), dim3(256), 0, s, p, SEG_MAX,
                            (uint16_t*)dk, (uint16_t*)dv, ws);
     } else {
         const int64_t blocks = p.Z * p.Hkv * p.K;
         if (blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
-        hipLaunchKernelGGL((gca_bwd_dkdv_mfma_kernel<D, false>), dim3((unsigned)blocks), dim3(128), 0, s, p,
-                           (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse, delta,
-                           dk, dv, ws);
+        if (D == 64)
+            hipLaunchKernelGGL((gca_bwd_dkdv2_mfma_kernel<D, false>), dim3((unsigned)blocks), dim3(128), 0, s, p,
+                               (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
+                               delta, dk, dv, ws);
+        else
+            hipLaunchKernelGGL((gca_bwd_dkdv_mfma_kernel<D, false>), dim3((unsigned)blocks), dim3(256), 0, s, p,
+                               (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
+                               delta, dk, dv, ws);
     }
     if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
     return (p.stages & GCA_STAGE_DW) ? launch_dw(p, delta, dw, s) : GCA_OK;

@@ -6,8 +6,9 @@
 // query tile) and walks the K retrieved chunks.  It has 2*GS wavefronts; wavefront w owns the
 // 32 query rows qb = w % 2 of query head w / 2.  Each retrieved chunk's K and V tiles
 // (64 x D bf16 each) are read from HBM once per workgroup with 16-byte coalesced loads,
-// staged in LDS (double buffered: the loads of chunk j+1 are issued before the math of chunk j),
-// and shared by all wavefronts.
+// staged in LDS (double buffered: the asynchronous loads of chunk j+1 are issued before the math of chunk j),
+// and shared by all wavefronts.  The copy is global_load_lds_dwordx4 (no staging registers); tiles are
+// unpadded and XOR-swizzled (gca_mfma.h).
 //
 // Per wavefront and chunk (v_mfma_f32_32x32x16_bf16, lane = (n = lane % 32, h = lane / 32)):
 //   S^T = K_j Q^T   A = K rows from LDS (16-byte reads), B = Q held in registers for the whole
@@ -24,28 +25,16 @@
 
 namespace gca {
 
-template <int D> struct FwdCfg {
-    static constexpr int KSTRIDE = D * 2 + 16;   // bytes per K row in LDS: 16-byte reads of 8 rows hit distinct banks
-    static constexpr int VSTRIDE = D * 2 + 32;   // bytes per V row in LDS: 4-row transposed patches hit distinct banks
-    static constexpr int KBYTES = 64 * KSTRIDE;
-    static constexpr int VBYTES = 64 * VSTRIDE;
-    static constexpr int BUF = KBYTES + VBYTES;
-};
-
 template <int D, int GS, bool INDEXED>
 __global__ void __launch_bounds__(128 * GS) __attribute__((amdgpu_waves_per_eu(2)))
 gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
                     const uint16_t* __restrict__ v, const int64_t* __restrict__ indices,
                     const void* __restrict__ w, int w_is_bf16, uint16_t* __restrict__ o, float* __restrict__ lse) {
-    using Cfg = FwdCfg<D>;
     constexpr int NT = 128 * GS;
     constexpr int KS = D / 16;                 // reduction steps of Q.K^T
     constexpr int DB = D / 32;                 // 32-wide dim blocks of O
-    constexpr int PIECES = 64 * D * 2 / 16;    // 16-byte pieces per tile
-    constexpr int LPT = PIECES / NT;           // pieces per thread per tile
-    constexpr int PPR = D * 2 / 16;            // pieces per row
-    static_assert(PIECES % NT == 0, "tile must split evenly over the workgroup");
-    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * Cfg::BUF];
+    constexpr int RB = D * 2, TILE = 64 * RB, BUF = 2 * TILE;   // K tile then V tile
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * BUF];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -83,57 +72,30 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
 
     const float c = p.sm_scale * LOG2E;
 
-    // staging: thread owns pieces tid + i*NT of each tile; piece = (row, 16-byte column)
-    u32x4 stage_k[LPT], stage_v[LPT];
-    int64_t goff[LPT];      // element offset of the piece inside a chunk (row stride applied)
-    int lds_koff[LPT], lds_voff[LPT];
-    {
-        const int64_t rs = p.indexed ? (int64_t)p.Hkv * D : (int64_t)D;
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) {
-            const int piece = tid + i * NT;
-            const int row = piece / PPR, col = piece % PPR;
-            goff[i] = row * rs + col * 8;
-            lds_koff[i] = row * Cfg::KSTRIDE + col * 16;
-            lds_voff[i] = row * Cfg::VSTRIDE + col * 16;
-        }
-    }
+    const TileLoader<D, NT> loader(tid, INDEXED ? p.Hkv * D : D);
     {
         int64_t rs;
-        const uint16_t* kj = chunk_base_n(p, k, indices, nseq, z, hk, 0, rs);
-        const uint16_t* vj = chunk_base_n(p, v, indices, nseq, z, hk, 0, rs);
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) {
-            stage_k[i] = *reinterpret_cast<const u32x4*>(kj + goff[i]);
-            stage_v[i] = *reinterpret_cast<const u32x4*>(vj + goff[i]);
-        }
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) {
-            *reinterpret_cast<u32x4*>(smem + lds_koff[i]) = stage_k[i];
-            *reinterpret_cast<u32x4*>(smem + Cfg::KBYTES + lds_voff[i]) = stage_v[i];
-        }
+        loader.issue(chunk_base_n(p, k, indices, nseq, z, hk, 0, rs), smem);
+        loader.issue(chunk_base_n(p, v, indices, nseq, z, hk, 0, rs), smem + TILE);
     }
+    wait_async_tiles();
     __syncthreads();
 
-    const int i16 = lane & 15;
-    const int dhalf = (lane >> 4) & 1;
+    const TrLane tr(lane);
+    const int fsw = swz(n);
 
     for (int j = 0; j < p.K; ++j) {
         const int buf = j & 1;
-        const bool more = (j + 1 < p.K);
-        if (more) {
+        if (j + 1 < p.K) {
+            // the other buffer was last read in iteration j-1, which every wavefront has left
             int64_t rs;
-            const uint16_t* kj = chunk_base_n(p, k, indices, nseq, z, hk, j + 1, rs);
-            const uint16_t* vj = chunk_base_n(p, v, indices, nseq, z, hk, j + 1, rs);
-#pragma unroll
-            for (int i = 0; i < LPT; ++i) {
-                stage_k[i] = *reinterpret_cast<const u32x4*>(kj + goff[i]);
-                stage_v[i] = *reinterpret_cast<const u32x4*>(vj + goff[i]);
-            }
+            unsigned char* nb = smem + (buf ^ 1) * BUF;
+            loader.issue(chunk_base_n(p, k, indices, nseq, z, hk, j + 1, rs), nb);
+            loader.issue(chunk_base_n(p, v, indices, nseq, z, hk, j + 1, rs), nb + TILE);
         }
 
-        const unsigned char* kb = smem + buf * Cfg::BUF;
-        const unsigned char* vb = kb + Cfg::KBYTES;
+        const unsigned char* kb = smem + buf * BUF;
+        const unsigned char* vb = kb + TILE;
 
         // ---- S^T = K Q^T : two 32-key tiles, keys in registers, query n in the lane
         f32x16 st[2];
@@ -141,10 +103,10 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
         for (int t = 0; t < 2; ++t) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) st[t][r] = 0.f;
-            const unsigned char* krow = kb + (32 * t + n) * Cfg::KSTRIDE + 16 * h;
+            const int rowoff = (32 * t + n) * RB;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const bf16x8 a = lds_read_b128(krow + 32 * ks);
+                const bf16x8 a = lds_read_b128(kb + rowoff + (((2 * ks + h) ^ fsw) << 4));
                 st[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qB[ks], st[t], 0, 0, 0);
             }
         }
@@ -185,22 +147,15 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
         // ---- O += P~ V
 #pragma unroll
         for (int t4 = 0; t4 < 4; ++t4) {
-            const unsigned char* vrow = vb + (16 * t4 + 4 * h + (i16 >> 2)) * Cfg::VSTRIDE + (16 * dhalf + 4 * (i16 & 3)) * 2;
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-                const bf16x8 b = lds_read_tr_pair(vrow + 64 * db, vrow + 64 * db + 8 * Cfg::VSTRIDE);
+                const int o0 = tr.off(t4, db, RB);
+                const bf16x8 b = lds_read_tr_pair(vb + o0, vb + o0 + 8 * RB);
                 oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pA[t4], b, oacc[db], 0, 0, 0);
             }
         }
 
-        if (more) {
-            unsigned char* nb = smem + (buf ^ 1) * Cfg::BUF;
-#pragma unroll
-            for (int i = 0; i < LPT; ++i) {
-                *reinterpret_cast<u32x4*>(nb + lds_koff[i]) = stage_k[i];
-                *reinterpret_cast<u32x4*>(nb + Cfg::KBYTES + lds_voff[i]) = stage_v[i];
-            }
-        }
+        wait_async_tiles();
         __syncthreads();
     }
 

@@ -63,6 +63,51 @@ struct TrLane {
     }
 };
 
+// Asynchronous global -> LDS copy of a 64 x D bf16 tile (rows `rs` elements apart in global memory)
+// into a swizzled LDS tile, with global_load_lds_dwordx4: lane l of an instruction deposits its 16 bytes
+// at lds_base + 16*l, so one instruction fills 1 KB = 64*16/RB consecutive tile rows.  The swizzle is
+// applied on the source side: the lane that writes physical piece pp of row r fetches logical piece
+// pp ^ swz(r).  Within a row the lanes still cover one contiguous 2*D-byte span of global memory.
+// No staging registers, no ds_write; completion is tracked by vmcnt (wait_async_tiles()).
+template <int D, int NT>
+struct TileLoader {
+    static constexpr int RB = D * 2;
+    static constexpr int PPR = RB / 16;             // 16-byte pieces per row
+    static constexpr int RPI = 64 / PPR;            // rows per instruction
+    static constexpr int NW = NT / 64;              // wavefronts sharing the copy
+    static constexpr int NI = 64 / RPI / NW;        // instructions per wavefront per tile
+    static_assert(NI >= 1 && NI * RPI * NW == 64, "tile must split evenly over the wavefronts");
+    int goff[NI];      // element offset of this lane's piece in instruction i
+    int wave;
+    __device__ __forceinline__ TileLoader(int tid, int rs) {
+        const int lane = tid & 63;
+        wave = tid >> 6;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int row = (i * NW + wave) * RPI + lane / PPR;
+            const int lp = (lane % PPR) ^ swz(row);
+            goff[i] = row * rs + lp * 8;
+        }
+    }
+    __device__ __forceinline__ void issue(const uint16_t* tile, unsigned char* lds_tile) const {
+        typedef __attribute__((address_space(3))) void lds_void;
+        typedef __attribute__((address_space(1))) const void gbl_void;
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+            __builtin_amdgcn_global_load_lds((gbl_void*)(tile + goff[i]), (lds_void*)(lds_tile + (i * NW + wave) * 1024), 16, 0, 0);
+    }
+};
+
+// 64 floats -> LDS (one wavefront, lane l writes element l)
+__device__ __forceinline__ void async_row64(const float* src, float* lds_dst, int lane) {
+    typedef __attribute__((address_space(3))) void lds_void;
+    typedef __attribute__((address_space(1))) const void gbl_void;
+    __builtin_amdgcn_global_load_lds((gbl_void*)(src + lane), (lds_void*)lds_dst, 4, 0, 0);
+}
+
+// all outstanding global_load_lds of this wavefront have landed (vmcnt = 0; other counters untouched)
+__device__ __forceinline__ void wait_async_tiles() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 // XCD-aware work order.  The hardware deals workgroups round-robin to the 8 XCDs (workgroup i runs
 // on XCD i % 8), each with its own L2.  Work items are numbered so that items sharing data are
 // consecutive ("logical" order); XCD x takes the contiguous range [x*per, (x+1)*per) of it, so the
