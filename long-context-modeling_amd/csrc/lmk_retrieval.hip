@@ -1,14 +1,16 @@
 // Landmark retrieval: scoring, strict-past mask, top-k selection, retrieval weights.
 //
-//   lmk_score   two kernels.  "scan": few query rows per sequence (decode): one wavefront per
-//               candidate landmark, 16-byte loads, wavefront reduction -- an HBM-bound stream
-//               over lmk_k.  "tile": many query rows (training/prefill): 32x32 output tiles,
-//               operands staged through LDS, tiles that are entirely masked are only filled.
+//   lmk_score   four kernels.  "scan_mfma": few query rows per sequence in bf16 (decode): the scan over
+//               lmk_k as a skinny GEMM, landmark rows loaded from HBM directly in MFMA operand form --
+//               an HBM-bound stream.  "scan": the same for fp32, one wavefront per candidate landmark,
+//               16-byte loads, wavefront reduction.  "mfma": many query rows in bf16 (training/prefill): 64x128 score blocks
+//               on the matrix cores, operands through swizzled LDS tiles.  "tile": the fp32 path and
+//               odd widths: 32x32 output tiles on the vector ALUs.  Fully masked blocks are only filled.
 //   lmk_topk    bitonic top-k in LDS over 64-bit keys (order-preserving image of the float in
 //               the high half, inverted index in the low half), so "higher value first, then
 //               lower index" is one unsigned compare and the result is unique.  Long rows are
 //               cut into segments (one workgroup each) whose winners a second launch merges.
-#include "gca_common.h"
+#include "gca_mfma.h"
 
 namespace gca {
 
@@ -40,7 +42,8 @@ __device__ __forceinline__ void unpack16(const uint4& raw, float (&out)[8]) {
 // One wavefront per candidate landmark e; all C (<= SCAN_MAX_C) query rows of the sequence
 // sit in LDS as floats.  Requires Dm % (16 / sizeof(T)) == 0.
 constexpr int SCAN_MAX_C = 4;
-constexpr int SCAN_EPW = 4;   // landmarks per wavefront per iteration (loads issued together)
+constexpr int SCAN_EPW = 8;   // landmarks per wavefront per step (loads issued together)
+constexpr int SCAN_STEPS = 4; // steps per wavefront: a workgroup scores 4 * SCAN_EPW * SCAN_STEPS landmarks
 
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -54,54 +57,214 @@ lmk_score_scan_kernel(lmk_desc d, const T* __restrict__ lq, const T* __restrict_
     __syncthreads();
     const float sqrt_hidden = sqrtf(d.hidden_size);
     const int nvec = Dm / VN;
-    const int64_t e0 = ((int64_t)blockIdx.x * 4 + wave) * SCAN_EPW;
-    float acc[SCAN_EPW][SCAN_MAX_C];
+    for (int step = 0; step < SCAN_STEPS; ++step) {
+        const int64_t e0 = (((int64_t)blockIdx.x * SCAN_STEPS + step) * 4 + wave) * SCAN_EPW;
+        if (e0 >= d.E) break;
+        float acc[SCAN_EPW][SCAN_MAX_C];
 #pragma unroll
-    for (int a = 0; a < SCAN_EPW; ++a)
+        for (int a = 0; a < SCAN_EPW; ++a)
 #pragma unroll
-        for (int c = 0; c < SCAN_MAX_C; ++c) acc[a][c] = 0.f;
+            for (int c = 0; c < SCAN_MAX_C; ++c) acc[a][c] = 0.f;
 
-    for (int iv = lane; iv < nvec; iv += 64) {
-        uint4 raw[SCAN_EPW];
+        for (int iv = lane; iv < nvec; iv += 64) {
+            u32x4 raw[SCAN_EPW];
 #pragma unroll
-        for (int a = 0; a < SCAN_EPW; ++a) {
-            const int64_t e = e0 + a;
-            raw[a] = make_uint4(0, 0, 0, 0);
-            if (e < d.E) raw[a] = *reinterpret_cast<const uint4*>(lk + (n * d.E + e) * Dm + (int64_t)iv * VN);
+            for (int a = 0; a < SCAN_EPW; ++a) {
+                const int64_t e = min(e0 + a, d.E - 1);          // the tail re-reads the last landmark
+                raw[a] = *reinterpret_cast<const u32x4*>(lk + (n * d.E + e) * Dm + (int64_t)iv * VN);
+            }
+#pragma unroll
+            for (int a = 0; a < SCAN_EPW; ++a) {
+                float kv[8];
+                if (VN == 8) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        kv[2 * i] = __uint_as_float(raw[a][i] << 16);
+                        kv[2 * i + 1] = __uint_as_float(raw[a][i] & 0xffff0000u);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) kv[i] = __uint_as_float(raw[a][i]);
+                }
+#pragma unroll
+                for (int c = 0; c < SCAN_MAX_C; ++c) {
+                    if (c < C) {
+#pragma unroll
+                        for (int i = 0; i < VN; ++i) acc[a][c] = fmaf(sq[c * Dm + iv * VN + i], kv[i], acc[a][c]);
+                    }
+                }
+            }
         }
 #pragma unroll
         for (int a = 0; a < SCAN_EPW; ++a) {
-            float kv[8];
-            if (VN == 8) {
-                unpack16(raw[a], kv);
-            } else {
-                kv[0] = __uint_as_float(raw[a].x); kv[1] = __uint_as_float(raw[a].y);
-                kv[2] = __uint_as_float(raw[a].z); kv[3] = __uint_as_float(raw[a].w);
-            }
 #pragma unroll
             for (int c = 0; c < SCAN_MAX_C; ++c) {
-                if (c < C) {
+                if (c >= C) continue;
+                float x = acc[a][c];
 #pragma unroll
-                    for (int i = 0; i < VN; ++i) acc[a][c] = fmaf(sq[c * Dm + iv * VN + i], kv[i], acc[a][c]);
+                for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off);
+                const int64_t e = e0 + a;
+                if (lane == 0 && e < d.E) {
+                    float r = finish_score<T>(x, sqrt_hidden);
+                    if (d.causal && !((d.E - C + c) > e)) r = -INFINITY;
+                    scores[(n * C + c) * d.E + e] = from_f<T>(r);
                 }
             }
         }
     }
+}
+
+// Decode scoring on the matrix cores (bf16, Dm % 16 == 0, at most SCANM_MAX_C query rows per sequence).
+// The scan over the cached landmarks is a skinny GEMM: scores[c, e] = sum_d lq[c, d] * lk[e, d].
+// Each wavefront takes 32 consecutive landmarks per step and loads their rows from HBM straight into
+// MFMA B-operand form (lane (n, h) holds landmark e0 + n, dims 16*ks + 8*h .. +7: 16-byte loads, every
+// byte of the row used once), the query rows wait in LDS as the A operand (rows >= C read as zero),
+// and 32 consecutive scores of a query row come out in one register across lanes 0-31: no unpacking,
+// no FMAs, no cross-lane reduction.  HBM-bound: E * Dm * 2 bytes per sequence.
+constexpr int SCANM_MAX_C = 32;
+constexpr int SCANM_UNROLL = 8;     // landmark-row loads in flight per lane
+
+__global__ void __launch_bounds__(256)
+lmk_score_scan_mfma_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const uint16_t* __restrict__ lk,
+                           uint16_t* __restrict__ scores, int steps) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char sqb[];   // C x Dm bf16
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n32 = lane & 31, h = lane >> 5;
+    const int64_t nb = blockIdx.y;
+    const int C = (int)d.C, Dm = d.Dm;
+    for (int i = tid; i < C * Dm / 8; i += 256)
+        reinterpret_cast<u32x4*>(sqb)[i] = reinterpret_cast<const u32x4*>(lq + nb * C * Dm)[i];
+    __syncthreads();
+    const float sqrt_hidden = sqrtf(d.hidden_size);
+    const int KS = Dm / 16;
+    const bool arow = n32 < C;
+    const unsigned char* aptr = sqb + (arow ? n32 : 0) * Dm * 2 + 16 * h;
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int step = 0; step < steps; ++step) {
+        const int64_t e0 = (((int64_t)blockIdx.x * steps + step) * 4 + wave) * 32;
+        if (e0 >= d.E) break;
+        const int64_t erow = min(e0 + n32, d.E - 1);                    // the tail re-reads the last landmark
+        const uint16_t* bptr = lk + (nb * d.E + erow) * Dm + 8 * h;
+        f32x16 acc;
 #pragma unroll
-    for (int a = 0; a < SCAN_EPW; ++a) {
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        int ks = 0;
+        for (; ks + SCANM_UNROLL <= KS; ks += SCANM_UNROLL) {
+            bf16x8 b[SCANM_UNROLL];
 #pragma unroll
-        for (int c = 0; c < SCAN_MAX_C; ++c) {
-            float x = acc[a][c];
+            for (int u = 0; u < SCANM_UNROLL; ++u) b[u] = *reinterpret_cast<const bf16x8*>(bptr + 16 * (ks + u));
 #pragma unroll
-            for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off);
-            const int64_t e = e0 + a;
-            if (lane == 0 && c < C && e < d.E) {
-                float r = finish_score<T>(x, sqrt_hidden);
-                if (d.causal && !((d.E - C + c) > e)) r = -INFINITY;
-                scores[(n * C + c) * d.E + e] = from_f<T>(r);
+            for (int u = 0; u < SCANM_UNROLL; ++u) {
+                const bf16x8 a = arow ? lds_read_b128(aptr + 32 * (ks + u)) : zero8;
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b[u], acc, 0, 0, 0);
+            }
+        }
+        for (; ks < KS; ++ks) {
+            const bf16x8 b = *reinterpret_cast<const bf16x8*>(bptr + 16 * ks);
+            const bf16x8 a = arow ? lds_read_b128(aptr + 32 * ks) : zero8;
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+        }
+        // register r is query row 8*(r/4) + 4*h + r%4, column = landmark e0 + n32
+        const int64_t e = e0 + n32;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int c = 8 * (r >> 2) + 4 * h + (r & 3);
+            if (c < C && e < d.E) {
+                float x = finish_score<bf16_t>(acc[r], sqrt_hidden);
+                if (d.causal && !((d.E - C + c) > e)) x = -INFINITY;
+                scores[(nb * C + c) * d.E + e] = f_to_bf16_bits(x);
             }
         }
     }
+}
+
+// Training / prefill scoring on the matrix cores (bf16, Dm % 64 == 0).  A workgroup of four wavefronts
+// computes a 64 (query landmarks) x 128 (candidate landmarks) block of scores; wavefront (wr, wc) owns
+// rows 32*wr.. and columns 64*wc...  The landmark width is consumed 64 dims at a time: the 64 x 64 A
+// sub-tile and the 128 x 64 B sub-tile go to LDS with asynchronous copies (double buffered, swizzled
+// like the attention tiles) and are read back as 16-byte MFMA operands.  Blocks that lie entirely in the
+// masked (future) region only write -inf.
+__global__ void __launch_bounds__(256)
+lmk_score_mfma_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const uint16_t* __restrict__ lk,
+                      uint16_t* __restrict__ scores) {
+    constexpr int TILE = 64 * 128;                // one 64-row x 64-dim sub-tile, bytes
+    constexpr int BUF = 3 * TILE;                 // A, B rows 0-63, B rows 64-127
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * BUF];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n32 = lane & 31, h = lane >> 5;
+    const int wr = wave >> 1, wc = wave & 1;
+    const int64_t nb = blockIdx.z;
+    const int64_t c0 = (int64_t)blockIdx.y * 64, e0 = (int64_t)blockIdx.x * 128;
+    const int64_t off = d.E - d.C;
+    const int64_t cmax = min(c0 + 63, d.C - 1);
+    const uint16_t NEG_INF = 0xff80;
+    if (d.causal && !((off + cmax) > e0)) {
+        for (int i = tid; i < 64 * 128; i += 256) {
+            const int64_t c = c0 + i / 128, e = e0 + i % 128;
+            if (c < d.C && e < d.E) scores[(nb * d.C + c) * d.E + e] = NEG_INF;
+        }
+        return;
+    }
+    // async copy plan: instruction i of this wavefront fills rows (i*4 + wave)*8 .. +7 of a sub-tile
+    int64_t aoff[2], b0off[2], b1off[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int row = (i * 4 + wave) * 8 + lane / 8;
+        const int lp = (lane % 8) ^ swz(row);
+        aoff[i] = (nb * d.C + min(c0 + row, d.C - 1)) * d.Dm + lp * 8;          // tail rows re-read the last row
+        b0off[i] = (nb * d.E + min(e0 + row, d.E - 1)) * d.Dm + lp * 8;
+        b1off[i] = (nb * d.E + min(e0 + 64 + row, d.E - 1)) * d.Dm + lp * 8;
+    }
+    typedef __attribute__((address_space(3))) void lds_void;
+    typedef __attribute__((address_space(1))) const void gbl_void;
+    auto issue = [&](int k0, int buf) {
+        unsigned char* base = smem + buf * BUF;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int lo = (i * 4 + wave) * 1024;
+            __builtin_amdgcn_global_load_lds((gbl_void*)(lq + aoff[i] + k0), (lds_void*)(base + lo), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gbl_void*)(lk + b0off[i] + k0), (lds_void*)(base + TILE + lo), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gbl_void*)(lk + b1off[i] + k0), (lds_void*)(base + 2 * TILE + lo), 16, 0, 0);
+        }
+    };
+    f32x16 acc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[t][r] = 0.f;
+    const int fsw = swz(n32);
+    const int nk = d.Dm / 64;
+    issue(0, 0);
+    wait_async_tiles();
+    __syncthreads();
+    for (int kc = 0; kc < nk; ++kc) {
+        const int buf = kc & 1;
+        if (kc + 1 < nk) issue((kc + 1) * 64, buf ^ 1);
+        const unsigned char* A = smem + buf * BUF + (32 * wr + n32) * 128;
+        const unsigned char* B = smem + buf * BUF + TILE + wc * TILE + n32 * 128;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const int po = ((2 * ks + h) ^ fsw) << 4;
+            const bf16x8 a = lds_read_b128(A + po);
+            acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, lds_read_b128(B + po), acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, lds_read_b128(B + 32 * 128 + po), acc[1], 0, 0, 0);
+        }
+        wait_async_tiles();
+        __syncthreads();
+    }
+    const float sqrt_hidden = sqrtf(d.hidden_size);
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int64_t c = c0 + 32 * wr + 8 * (r >> 2) + 4 * h + (r & 3);
+            const int64_t e = e0 + 64 * wc + 32 * t + n32;
+            if (c < d.C && e < d.E) {
+                float x = finish_score<bf16_t>(acc[t][r], sqrt_hidden);
+                if (d.causal && !((off + c) > e)) x = -INFINITY;
+                scores[(nb * d.C + c) * d.E + e] = f_to_bf16_bits(x);
+            }
+        }
 }
 
 // 32x32 output tile per workgroup, 2x2 outputs per thread, Dm consumed in steps of 32.
@@ -158,12 +321,27 @@ static int launch_score_t(const lmk_desc& d, const void* lq, const void* lk, voi
     constexpr int VN = Vec16<T>::N;
     const bool aligned = (((uintptr_t)lk) % 16 == 0) && (d.Dm % VN == 0);
     const size_t lds = (size_t)d.C * d.Dm * sizeof(float);
-    if (d.C <= SCAN_MAX_C && aligned && lds <= 48 * 1024 && d.N <= 65535) {
-        const int64_t per_block = 4 * SCAN_EPW;
+    if (sizeof(T) == 2 && d.C <= SCANM_MAX_C && d.Dm % 16 == 0 && (((uintptr_t)lk | (uintptr_t)lq) % 16 == 0) &&
+        (size_t)d.C * d.Dm * 2 <= 64 * 1024 && d.N <= 65535) {
+        // aim at >= 2048 workgroups; each step of a workgroup covers 128 landmarks
+        const int64_t units = (d.E + 127) / 128;
+        int steps = (int)((units * d.N + 2047) / 2048);
+        steps = steps < 1 ? 1 : (steps > 8 ? 8 : steps);
+        const int64_t bx = (units + steps - 1) / steps;
+        if (bx > 0x7fffffffLL) return GCA_ERR_SHAPE;
+        hipLaunchKernelGGL(lmk_score_scan_mfma_kernel, dim3((unsigned)bx, (unsigned)d.N), dim3(256), (size_t)d.C * d.Dm * 2, s, d,
+                           (const uint16_t*)lq, (const uint16_t*)lk, (uint16_t*)scores, steps);
+    } else if (d.C <= SCAN_MAX_C && aligned && lds <= 48 * 1024 && d.N <= 65535) {
+        const int64_t per_block = 4 * SCAN_EPW * SCAN_STEPS;
         const int64_t bx = (d.E + per_block - 1) / per_block;
         if (bx > 0x7fffffffLL) return GCA_ERR_SHAPE;
         hipLaunchKernelGGL((lmk_score_scan_kernel<T>), dim3((unsigned)bx, (unsigned)d.N), dim3(256), lds, s, d,
                            (const T*)lq, (const T*)lk, (T*)scores);
+    } else if (sizeof(T) == 2 && d.Dm % 64 == 0 && (((uintptr_t)lk | (uintptr_t)lq) % 16 == 0) && d.C >= 32) {
+        const int64_t bx = (d.E + 127) / 128, by = (d.C + 63) / 64;
+        if (bx > 0x7fffffffLL || by > 65535 || d.N > 65535) return GCA_ERR_SHAPE;
+        hipLaunchKernelGGL(lmk_score_mfma_kernel, dim3((unsigned)bx, (unsigned)by, (unsigned)d.N), dim3(256), 0, s, d,
+                           (const uint16_t*)lq, (const uint16_t*)lk, (uint16_t*)scores);
     } else {
         const int64_t bx = (d.E + 31) / 32, by = (d.C + 31) / 32;
         if (bx > 0x7fffffffLL || by > 65535 || d.N > 65535) return GCA_ERR_SHAPE;
