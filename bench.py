@@ -105,6 +105,92 @@ def kernel_times(torch, q, ck, cv, idx, w, do, sm_scale, sm_n, iters):
     return times
 
 
+def other_configs(torch, dev, seed):
+    """BASELINE configs 3, 4, 5 on the same GPU: absolute tokens/s and the fraction of the binding
+    (HBM) roofline from the stream-model bytes.  Forward-only configs time scoring + top-k + forward."""
+    import gca_hip
+    g = torch.Generator(device=dev).manual_seed(seed + 1)
+
+    def rn(*shape, scale=1.0):
+        return (torch.randn(*shape, device=dev, generator=g) * scale).bfloat16()
+
+    out = {}
+    # ---- config 4: GQA, wider heads, fwd+bwd.  Retrieval score logits ~ N(0,1) are given directly.
+    N, C, Hq, Hkv, S, d, K = 4, 512, 32, 8, 64, 128, 16
+    Z = N * (C - 1)
+    q = rn(Z, Hq, S, d, scale=0.35).requires_grad_(True)
+    do = rn(Z, Hq, S, d)
+    ck = rn(N, C, S, Hkv * d, scale=0.35).requires_grad_(True)
+    cv = rn(N, C, S, Hkv * d, scale=0.35).requires_grad_(True)
+    scores = torch.randn(N, C, C, device=dev, generator=g).bfloat16()
+
+    def step4():
+        indices, weights = gca_hip.landmark_topk(scores, K)
+        idx = indices[:, :-1].reshape(Z, K).contiguous()
+        w = weights[:, :-1].reshape(Z, K).contiguous().requires_grad_(True)
+        o = gca_hip.attention_indexed(q, ck, cv, idx, w, 1.0 / math.sqrt(d), 0.0)
+        return torch.autograd.grad(o, (q, ck, cv, w), do)
+
+    t = event_time(torch, step4, 5) * 1e-3
+    tokens = N * C * S
+    e = 2
+    nbytes = (2 * Hq * d * e + 2 * K * Hkv * d * e + 4 * Hq * K) + (3 * Hq * d * e + 4 * Hq * K + 2 * K * Hkv * d * e + 2 * K * Hkv * d * 4)
+    flops = 14 * Hq * K * S * d
+    t_roof = max(nbytes * tokens / (HBM_PEAK_GBS * 1e9), flops * tokens / 2.5e15)
+    out["cfg4_gqa_d128_fwd_bwd"] = {"tokens_per_s": round(tokens / t, 1), "ms": round(t * 1e3, 3),
+                                    "frac_of_binding_roofline": round(t_roof / t, 4), "bound": "hbm",
+                                    "algorithmic_TFLOP_per_s": round(flops * tokens / t / 1e12, 1)}
+    del q, do, ck, cv, scores
+
+    # ---- config 3: 1M-token prefill, forward only, one needle chunk with a 4x landmark
+    N, C, H, S, d, K = 1, 16384, 12, 64, 64, 8
+    Z = C - 1
+    q = rn(Z, H, S, d, scale=0.5)
+    ck, cv = rn(N, C, S, H * d, scale=0.5), rn(N, C, S, H * d, scale=0.5)
+    lk = (ck.float().mean(2) + 0.1 * torch.randn(N, C, H * d, device=dev, generator=g)).bfloat16()
+    lq = rn(N, C, H * d)
+    needle = 4321
+    lk[0, needle] = lk[0, needle] * 4 + lq[0, -1] * 0      # 4x norm at a fixed position
+    lq = (lq + 0.5 * lk[0, needle]).bfloat16()            # queries correlate with the needle
+
+    def step3():
+        _, indices, weights = gca_hip.landmark_retrieve(lq, lk, K, H * d)
+        idx = indices[:, :-1].reshape(Z, K).contiguous()
+        w = weights[:, :-1].reshape(Z, K).contiguous()
+        return gca_hip.gca_kv_cache_indexed(q, ck, cv, idx, w, 0.125, 1.0), indices
+
+    _, indices = step3()
+    hit = (indices[0, needle + 1:] == needle).any(-1).float().mean().item()
+    t = event_time(torch, lambda: step3(), 3, 1) * 1e-3
+    tokens = N * C * S
+    nbytes = (2 * H * d * e + 2 * K * H * d * e + 4 * H * K) * tokens + 2 * N * C * H * d * e
+    out["cfg3_prefill_1M_fwd"] = {"tokens_per_s": round(tokens / t, 1), "ms": round(t * 1e3, 3),
+                                  "frac_of_binding_roofline": round(nbytes / (HBM_PEAK_GBS * 1e9) / t, 4), "bound": "hbm",
+                                  "needle_selected_by_later_rows": round(hit, 4)}
+    del q, ck, cv, lk, lq
+
+    # ---- config 5: one decode chunk (64 new tokens) per sequence against a long cache
+    for name, N, E in (("cfg5a_decode_B1_16M", 1, 262144), ("cfg5b_decode_B64_64K", 64, 1024)):
+        H, S, d, K = 12, 64, 64, 8
+        ck, cv = rn(N, E, S, H * d, scale=0.5), rn(N, E, S, H * d, scale=0.5)
+        lk, lq = rn(N, E, H * d), rn(N, 1, H * d)
+        q = rn(N, H, S, d, scale=0.5)
+
+        def step5():
+            _, indices, weights = gca_hip.landmark_retrieve(lq, lk, K, H * d)
+            return gca_hip.gca_kv_cache_indexed(q, ck, cv, indices.view(N, K), weights.view(N, K), 0.125, 1.0)
+
+        t = event_time(torch, step5, 20, 3) * 1e-3
+        nbytes = N * E * H * d * e + N * (2 * K * S * H * d * e + 2 * H * S * d * e)
+        out[name] = {"new_tokens_per_s": round(N * S / t, 1), "us": round(t * 1e6, 2),
+                     "frac_of_binding_roofline": round(nbytes / (HBM_PEAK_GBS * 1e9) / t, 4), "bound": "hbm",
+                     "scan_GB_per_s": None}
+        t_scan = event_time(torch, lambda: gca_hip.landmark_scores(lq, lk, H * d), 20, 3) * 1e-3
+        out[name]["scan_GB_per_s"] = round(N * E * H * d * e / t_scan / 1e9, 1)
+        del ck, cv, lk, lq, q
+    return out
+
+
 def cpu_baseline(torch, budget_s=12.0):
     """CPU oracle at BASELINE.json config 1 (fp32, B=2, H=4, d=64, L=1024, chunk 64, top-k 4, softmax1 on):
     retrieval + forward + autograd backward, median over the iterations that fit the budget."""
@@ -146,6 +232,8 @@ def main():
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--sm-n", type=float, default=1.0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--all-configs", action="store_true",
+                    help="also time BASELINE configs 3, 4 and 5 (adds an other_configs object to the JSON line)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 1 GiB device-to-device copy (a kernel of known traffic, for scaling "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
@@ -224,6 +312,10 @@ def main():
                    "softmax_off_by_one": args.sm_n},
         "roofline": roofline,
     }
+    if args.all_configs:
+        del q, ck, cv, lq, lk, do
+        torch.cuda.empty_cache()
+        out["other_configs"] = other_configs(torch, dev, args.seed)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(out), flush=True)

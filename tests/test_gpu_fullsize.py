@@ -1,0 +1,178 @@
+"""Full-size checks at BASELINE.json's shapes, through properties that do not need the CPU oracle:
+agreement of the MFMA kernels with the independent generic (fp32-arithmetic) kernels, linearity in V,
+invariance under a permutation of the retrieval slots, the dw / delta identity, indexed == gathered,
+the needle of config 3, and scoring / top-k against torch's own device ops.  Tolerance for bf16
+comparisons: max |a-b| / max |b| <= 2e-2."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _rel(a, b):
+    a, b = a.float(), b.float()
+    return ((a - b).abs().max() / b.abs().max().clamp_min(1e-30)).item()
+
+
+def _cfg2(seed=0, N=8, C=256, H=12, S=64, d=64, K=8):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    Z = N * (C - 1)
+    q = (torch.randn(Z, H, S, d, device=DEV, generator=g) * 0.5).bfloat16()
+    ck = (torch.randn(N, C, S, H * d, device=DEV, generator=g) * 0.5).bfloat16()
+    cv = (torch.randn(N, C, S, H * d, device=DEV, generator=g) * 0.5).bfloat16()
+    lk = (ck.float().mean(2) + 0.1 * torch.randn(N, C, H * d, device=DEV, generator=g)).bfloat16()
+    lq = torch.randn(N, C, H * d, device=DEV, generator=g).bfloat16()
+    do = torch.randn(Z, H, S, d, device=DEV, generator=g).bfloat16()
+    return q, ck, cv, lq, lk, do
+
+
+def _run_indexed(q, ck, cv, idx, w, do, path, sm_n=1.0):
+    import gca_hip
+    from gca_hip import gca as G
+    old = G.kernel_path
+    G.kernel_path = path
+    try:
+        a = [t.detach().clone().requires_grad_(True) for t in (q, ck, cv, w)]
+        o = gca_hip.attention_indexed(a[0], a[1], a[2], idx, a[3], 0.125, sm_n)
+        grads = torch.autograd.grad(o, a, do)
+    finally:
+        G.kernel_path = old
+    return (o.detach(),) + tuple(grads)
+
+
+def test_cfg2_mfma_vs_generic_and_invariants():
+    import gca_hip
+    q, ck, cv, lq, lk, do = _cfg2()
+    N, C, S, Dm = ck.shape
+    Z, H, _, d = q.shape
+    K = 8
+    _, indices, weights = gca_hip.landmark_retrieve(lq, lk, K, Dm)
+    idx = indices[:, :-1].reshape(Z, K).contiguous()
+    w = weights[:, :-1].reshape(Z, K).contiguous()
+    assert (idx[w > 0] < (torch.arange(Z, device=DEV) % (C - 1) + 1)[:, None].expand(Z, K)[w > 0]).all()   # strictly past
+    mf = _run_indexed(q, ck, cv, idx, w, do, "mfma")
+    ge = _run_indexed(q, ck, cv, idx, w, do, "generic")
+    for name, a, b in zip(("o", "dq", "dk_cache", "dv_cache", "dw"), mf, ge):
+        assert torch.isfinite(a.float()).all(), name
+        assert _rel(a, b) <= 2e-2, (name, _rel(a, b))
+    o, dq, dkc, dvc, dw = mf
+    # sum_j w_j dw_j = sum_{h,m} <O, dO> per query chunk (both sides are sum_j w_j D_j)
+    lhs = (w * dw.float()).sum(-1)
+    rhs = (o.float() * do.float()).sum((1, 2, 3))
+    assert ((lhs - rhs).abs().max() / rhs.abs().max()).item() <= 2e-2
+    # the first query chunk of every sequence retrieved nothing but chunk 0; chunks nobody retrieved get zero gradient
+    used = torch.zeros(N, C, dtype=torch.bool, device=DEV)
+    used.view(-1)[(idx + (torch.arange(Z, device=DEV) // (C - 1) * C)[:, None]).view(-1)] = True
+    assert dkc[~used].abs().max() == 0 and dvc[~used].abs().max() == 0
+    # permuting the retrieval slots of every row changes nothing (slots are summed)
+    perm = torch.randperm(K, device=DEV)
+    o2 = gca_hip.gca_kv_cache_indexed(q, ck, cv, idx[:, perm].contiguous(), w[:, perm].contiguous(), 0.125, 1.0)
+    assert _rel(o2, o) <= 1e-2
+    # linearity in V: f(V1 + V2) = f(V1) + f(V2)
+    cv2 = torch.randn_like(cv) * 0.5
+    o_a = gca_hip.gca_kv_cache_indexed(q, ck, cv2, idx, w, 0.125, 1.0)
+    o_s = gca_hip.gca_kv_cache_indexed(q, ck, (cv.float() + cv2.float()).bfloat16(), idx, w, 0.125, 1.0)
+    assert _rel(o_s, o.float() + o_a.float()) <= 2e-2
+
+
+def test_cfg2_indexed_equals_gathered():
+    import gca_hip
+    q, ck, cv, lq, lk, do = _cfg2(seed=1, N=2)
+    N, C, S, Dm = ck.shape
+    Z, H, _, d = q.shape
+    K = 8
+    _, indices, weights = gca_hip.landmark_retrieve(lq, lk, K, Dm)
+    idx = indices[:, :-1].reshape(Z, K).contiguous()
+    w = weights[:, :-1].reshape(Z, K).contiguous()
+    kg, vg, wg = gca_hip.gather_chunks(ck, cv, indices, weights, H)
+    kg.requires_grad_(True); vg.requires_grad_(True)
+    qg = q.clone().requires_grad_(True)
+    og = gca_hip.attention(qg, kg, vg, wg, 0.125, 1.0)
+    dqg, dkg, dvg = torch.autograd.grad(og, (qg, kg, vg), do)
+    o, dq, dkc, dvc, dw = _run_indexed(q, ck, cv, idx, w, do, "mfma")
+    assert _rel(o, og) <= 1e-2 and _rel(dq, dqg) <= 1e-2
+    # scatter-add the gathered gradients back into the cache layout
+    ref = torch.zeros(N * C, S, H, d, device=DEV)
+    flat = (idx + (torch.arange(Z, device=DEV) // (C - 1) * C)[:, None]).view(-1)
+    ref.index_add_(0, flat, dkg.float().permute(0, 2, 3, 1, 4).reshape(Z * K, S, H, d))
+    assert _rel(dkc.view(N * C, S, H, d), ref) <= 2e-2
+
+
+def test_cfg4_geometry_mfma_vs_generic():
+    # 32 query heads over 8 kv heads, d=128, top-k 16 at a reduced batch
+    import gca_hip
+    N, C, Hq, Hkv, S, d, K = 1, 64, 32, 8, 64, 128, 16
+    g = torch.Generator(device=DEV).manual_seed(3)
+    Z = N * (C - 1)
+    q = (torch.randn(Z, Hq, S, d, device=DEV, generator=g) * 0.35).bfloat16()
+    ck = (torch.randn(N, C, S, Hkv * d, device=DEV, generator=g) * 0.35).bfloat16()
+    cv = (torch.randn(N, C, S, Hkv * d, device=DEV, generator=g) * 0.35).bfloat16()
+    do = torch.randn(Z, Hq, S, d, device=DEV, generator=g).bfloat16()
+    scores = torch.randn(N, C, C, device=DEV, generator=g).bfloat16()
+    indices, weights = gca_hip.landmark_topk(scores, K)
+    idx = indices[:, :-1].reshape(Z, K).contiguous()
+    w = weights[:, :-1].reshape(Z, K).contiguous()
+    import gca_hip.gca as G
+    mf = _run_indexed(q, ck, cv, idx, w, do, "mfma", sm_n=0.0)
+    ge = _run_indexed(q, ck, cv, idx, w, do, "generic", sm_n=0.0)
+    for name, a, b in zip(("o", "dq", "dk_cache", "dv_cache", "dw"), mf, ge):
+        assert _rel(a, b) <= 2e-2, (name, _rel(a, b))
+
+
+def test_cfg3_needle_over_long_candidate_list():
+    # 16384 chunks, one needle landmark with 4x norm: every later row must retrieve it first
+    import gca_hip
+    N, C, Dm, K = 1, 16384, 768, 8
+    g = torch.Generator(device=DEV).manual_seed(5)
+    lk = torch.randn(N, C, Dm, device=DEV, generator=g).bfloat16()
+    needle = 4321
+    direction = lk[0, needle].float()
+    lk[0, needle] = (4 * direction).bfloat16()
+    lq = (torch.randn(N, C, Dm, device=DEV, generator=g) + 0.5 * direction).bfloat16()
+    scores, indices, weights = gca_hip.landmark_retrieve(lq, lk, K, Dm)
+    assert (indices[0, needle + 1:, 0] == needle).all()
+    assert not (indices[0, :needle + 1] == needle)[weights[0, :needle + 1] > 0].any()        # never before it exists
+    # scores agree with a device matmul; selection is the canonical top-k of the kernel's own scores
+    rows = torch.arange(C - 64, C, device=DEV)
+    ref = (lq[0, rows].float() @ lk[0].float().T) / math.sqrt(Dm)
+    got = scores[0, rows].float()
+    vis = torch.arange(C, device=DEV)[None, :] < rows[:, None]
+    assert torch.isinf(got[~vis]).all()
+    assert ((got[vis] - ref[vis]).abs().max() / ref[vis].abs().max()).item() <= 2e-2
+    srt = torch.sort(got, dim=-1, descending=True, stable=True)
+    assert torch.equal(indices[0, rows], srt.indices[:, :K])
+    assert (weights.sum(-1)[0, 1:] - 1).abs().max() <= 1e-5 and weights[0, 0].abs().max() == 0
+
+
+@pytest.mark.parametrize("N,E", [(1, 262144), (64, 1024)])
+def test_cfg5_decode_scan_topk(N, E):
+    import gca_hip
+    Dm, K = 768, 8
+    g = torch.Generator(device=DEV).manual_seed(6)
+    lk = torch.randn(N, E, Dm, device=DEV, generator=g).bfloat16()
+    lq = torch.randn(N, 1, Dm, device=DEV, generator=g).bfloat16()
+    scores, indices, weights = gca_hip.landmark_retrieve(lq, lk, K, Dm)
+    ref = torch.einsum('ncd,ned->nce', lq.float(), lk.float()) / math.sqrt(Dm)
+    got = scores.float()
+    assert torch.isinf(got[:, 0, -1]).all()                       # the new chunk does not see itself
+    assert ((got[:, :, :-1] - ref[:, :, :-1]).abs().max() / ref.abs().max()).item() <= 2e-2
+    srt = torch.sort(got, dim=-1, descending=True, stable=True)
+    assert torch.equal(indices, srt.indices[..., :K])
+    assert (weights.sum(-1) - 1).abs().max() <= 1e-5
+    # decode attention over the retrieved chunks: MFMA kernel vs generic kernel
+    H, S, d = 12, 64, 64
+    ck = (torch.randn(N, E, S, H * d, device=DEV, generator=g) * 0.5).bfloat16() if N * E <= 65536 else None
+    if ck is not None:
+        cv = (torch.randn(N, E, S, H * d, device=DEV, generator=g) * 0.5).bfloat16()
+        q = (torch.randn(N, H, S, d, device=DEV, generator=g) * 0.5).bfloat16()
+        import gca_hip.gca as G
+        a = gca_hip.gca_kv_cache_indexed(q, ck, cv, indices.view(N, K), weights.view(N, K), 0.125, 1.0)
+        G.kernel_path = "generic"
+        try:
+            b = gca_hip.gca_kv_cache_indexed(q, ck, cv, indices.view(N, K), weights.view(N, K), 0.125, 1.0)
+        finally:
+            G.kernel_path = "auto"
+        assert _rel(a, b) <= 2e-2
