@@ -28,13 +28,16 @@
 //    partial tiles; a small reduce launch adds those up in segment order.
 //
 // dw[z, j] = sum over heads and rows of delta (shared launch_dw).
+#include <cstdlib>
 #include "gca_mfma.h"
 #include "gca_lists.h"
 
 namespace gca {
 
 
-constexpr int SEG_MAX = 16;   // references per dkdv workgroup in the indexed form
+static int seg_max_from_env() { const char* e = getenv("GCA_SEG_MAX"); const int v = e ? atoi(e) : 0; return v > 0 ? v : 32; }
+// references per dkdv workgroup in the indexed form (GCA_SEG_MAX overrides, for tuning)
+static const int SEG_MAX = seg_max_from_env();
 
 // ------------------------------------------------------------------------------------------- dq
 
@@ -185,7 +188,7 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
                          const uint16_t* __restrict__ v, const void* __restrict__ w, int w_is_bf16,
                          const uint16_t* __restrict__ dout, const float* __restrict__ lse,
                          const float* __restrict__ delta, void* __restrict__ dk_out, void* __restrict__ dv_out,
-                         ListWs ws) {
+                         ListWs ws, int seg_per) {
     constexpr int NT = 128;
     constexpr int KS = D / 16, DB = D / 32;
     constexpr int RB = D * 2, TILE = 64 * RB, BUF = 2 * TILE;   // Q tile then dO tile
@@ -205,9 +208,17 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
     const uint16_t* vt;
     int64_t rs, out_off;     // key-row stride of the tile; element offset of the tile in the output
     if (INDEXED) {
-        const int seg = blockIdx.x / p.Hkv;
-        hk = blockIdx.x % p.Hkv;
-        if (seg >= ws.nseg[0]) return;
+        // (sequence, kv head) pairs are dealt round-robin to the XCDs (workgroup b runs on XCD b % 8), so the
+        // Q / dO tiles a pair's chunks keep re-reading stay in one L2; seg_per = segment slots per sequence.
+        const int64_t idx = blockIdx.x / NUM_XCD;
+        const int64_t pair = (idx / seg_per) * NUM_XCD + blockIdx.x % NUM_XCD;
+        if (pair >= p.N * p.Hkv) return;
+        const int64_t nseq = pair / p.Hkv;
+        hk = (int)(pair % p.Hkv);
+        const int seg_lo = ws.seg_base[nseq * p.C];
+        const int seg_hi = nseq + 1 < p.N ? ws.seg_base[(nseq + 1) * p.C] : ws.nseg[0];
+        const int seg = seg_lo + (int)(idx % seg_per);
+        if (seg >= seg_hi) return;
         const int64_t cc = ws.seg_chunk[seg];
         list0 = ws.seg_start[seg];
         nunits = ws.seg_len[seg] * p.G * (p.Q_CTX / 64);
@@ -383,7 +394,7 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
                          const uint16_t* __restrict__ v, const void* __restrict__ w, int w_is_bf16,
                          const uint16_t* __restrict__ dout, const float* __restrict__ lse,
                          const float* __restrict__ delta, void* __restrict__ dk_out, void* __restrict__ dv_out,
-                         ListWs ws) {
+                         ListWs ws, int seg_per) {
     constexpr int NT = 256;
     constexpr int KS = D / 16, DB = D / 32, DBH = DB / 2;
     constexpr int RB = D * 2, TILE = 64 * RB, BUF = 2 * TILE;   // Q tile then dO tile
@@ -404,9 +415,17 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
     const uint16_t* vt;
     int64_t rs, out_off;     // key-row stride of the tile; element offset of the tile in the output
     if (INDEXED) {
-        const int seg = blockIdx.x / p.Hkv;
-        hk = blockIdx.x % p.Hkv;
-        if (seg >= ws.nseg[0]) return;
+        // (sequence, kv head) pairs are dealt round-robin to the XCDs (workgroup b runs on XCD b % 8), so the
+        // Q / dO tiles a pair's chunks keep re-reading stay in one L2; seg_per = segment slots per sequence.
+        const int64_t idx = blockIdx.x / NUM_XCD;
+        const int64_t pair = (idx / seg_per) * NUM_XCD + blockIdx.x % NUM_XCD;
+        if (pair >= p.N * p.Hkv) return;
+        const int64_t nseq = pair / p.Hkv;
+        hk = (int)(pair % p.Hkv);
+        const int seg_lo = ws.seg_base[nseq * p.C];
+        const int seg_hi = nseq + 1 < p.N ? ws.seg_base[(nseq + 1) * p.C] : ws.nseg[0];
+        const int seg = seg_lo + (int)(idx % seg_per);
+        if (seg >= seg_hi) return;
         const int64_t cc = ws.seg_chunk[seg];
         list0 = ws.seg_start[seg];
         nunits = ws.seg_len[seg] * p.G * (p.Q_CTX / 64);
@@ -651,20 +670,23 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
     if (!(p.stages & GCA_STAGE_DKDV)) return (p.stages & GCA_STAGE_DW) ? launch_dw(p, delta, dw, s) : GCA_OK;
 
     ListWs ws = {};
+    const int seg_per0 = 0;
     if (p.indexed) {
         // the list workspace follows delta
         ws = list_carve(p, SEG_MAX, (char*)delta + delta_bytes(p));
         if ((rc = list_build(p, SEG_MAX, idx, ws, s)) != GCA_OK) return rc;
-        const int64_t blocks = list_seg_bound(p, SEG_MAX) * p.Hkv;
+        // segment slots per sequence: every chunk has one segment, plus one per SEG_MAX references
+        const int seg_per = (int)(p.C + (p.zpn * p.K + SEG_MAX - 1) / SEG_MAX);
+        const int64_t blocks = (p.N * p.Hkv + NUM_XCD - 1) / NUM_XCD * NUM_XCD * seg_per;
         if (blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
         if (D == 64)
             hipLaunchKernelGGL((gca_bwd_dkdv2_mfma_kernel<D, true>), dim3((unsigned)blocks), dim3(128), 0, s, p,
                                (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
-                               delta, dk, dv, ws);
+                               delta, dk, dv, ws, seg_per);
         else
             hipLaunchKernelGGL((gca_bwd_dkdv_mfma_kernel<D, true>), dim3((unsigned)blocks), dim3(256), 0, s, p,
                                (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
-                               delta, dk, dv, ws);
+                               delta, dk, dv, ws, seg_per);
         hipLaunchKernelGGL((gca_bwd_dkdv_reduce_kernel<D>), dim3((unsigned)(p.N * p.C * p.Hkv)), dim3(256), 0, s, p, SEG_MAX,
                            (uint16_t*)dk, (uint16_t*)dv, ws);
     } else {
@@ -673,11 +695,11 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
         if (D == 64)
             hipLaunchKernelGGL((gca_bwd_dkdv2_mfma_kernel<D, false>), dim3((unsigned)blocks), dim3(128), 0, s, p,
                                (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
-                               delta, dk, dv, ws);
+                               delta, dk, dv, ws, seg_per0);
         else
             hipLaunchKernelGGL((gca_bwd_dkdv_mfma_kernel<D, false>), dim3((unsigned)blocks), dim3(256), 0, s, p,
                                (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
-                               delta, dk, dv, ws);
+                               delta, dk, dv, ws, seg_per0);
     }
     if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
     return (p.stages & GCA_STAGE_DW) ? launch_dw(p, delta, dw, s) : GCA_OK;
