@@ -152,6 +152,17 @@ int lmk_score_topk(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, c
                    void* scores, int64_t* indices, float* weights,
                    void* workspace, size_t workspace_bytes, void* stream);
 
+/* Bytes of scratch lmk_weights_bwd needs. */
+size_t lmk_weights_bwd_workspace_bytes(const lmk_desc* desc);
+
+/* Gradient of the retrieval weights w.r.t. both landmark embeddings, the top-k selection held fixed:
+ * given dweights (N, C, kk) float it returns dlmk_q (N, C, Dm) and dlmk_k (N, E, Dm) in desc.dtype.
+ * Replaces what autograd runs backwards through model/DRT.py:626-627 (softmax, gather) and :612
+ * (einsum / sqrt(hidden)); deterministic (no atomics). */
+int lmk_weights_bwd(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, const int64_t* indices,
+                    const float* weights, const float* dweights, void* dlmk_q, void* dlmk_k,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -147,4 +147,19 @@ int lmk_score_topk(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, c
     return lmk_topk(desc, scores, noise, indices, weights, workspace, workspace_bytes, stream);
 }
 
+size_t lmk_weights_bwd_workspace_bytes(const lmk_desc* desc) {
+    if (check_lmk(desc) != GCA_OK) return 0;
+    return lmk_bwd_ws_bytes(*desc);
+}
+
+int lmk_weights_bwd(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, const int64_t* indices,
+                    const float* weights, const float* dweights, void* dlmk_q, void* dlmk_k,
+                    void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_lmk(desc);
+    if (rc != GCA_OK) return rc;
+    if (!lmk_q || !lmk_k || !indices || !weights || !dweights || !dlmk_q || !dlmk_k) return GCA_ERR_NULL;
+    return launch_lmk_bwd(*desc, lmk_q, lmk_k, indices, weights, dweights, dlmk_q, dlmk_k, workspace, workspace_bytes,
+                          (hipStream_t)stream);
+}
+
 }  // extern "C"

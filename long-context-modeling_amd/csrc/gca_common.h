@@ -94,6 +94,9 @@ int launch_lmk_score(const lmk_desc& d, const void* lq, const void* lk, void* sc
 int launch_lmk_topk(const lmk_desc& d, const void* scores, const void* noise, int64_t* indices, float* weights,
                     void* ws, size_t ws_bytes, hipStream_t s);
 size_t lmk_topk_ws_bytes(const lmk_desc& d);
+size_t lmk_bwd_ws_bytes(const lmk_desc& d);
+int launch_lmk_bwd(const lmk_desc& d, const void* lq, const void* lk, const int64_t* idx, const float* w,
+                   const float* dw, void* dlq, void* dlk, void* wsp, size_t ws_bytes, hipStream_t s);
 size_t bwd_workspace_bytes(const gca_desc& d, bool indexed);
 int launch_dw(const Params& p, const float* delta, float* dw, hipStream_t s);
 // bytes of the per-chunk row sums D_j at the start of the backward workspace (256-byte multiple)

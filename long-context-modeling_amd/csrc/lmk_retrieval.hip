@@ -11,6 +11,7 @@
 //               lower index" is one unsigned compare and the result is unique.  Long rows are
 //               cut into segments (one workgroup each) whose winners a second launch merges.
 #include "gca_mfma.h"
+#include "gca_lists.h"
 
 namespace gca {
 
@@ -589,6 +590,97 @@ int launch_lmk_topk(const lmk_desc& d, const void* scores, const void* noise, in
     if (need > 0 && (ws == nullptr || ws_bytes < need)) return GCA_ERR_WORKSPACE;
     if (d.dtype == GCA_F32) return launch_topk_t<float>(d, pl, scores, noise, indices, weights, ws, s);
     if (d.dtype == GCA_BF16) return launch_topk_t<bf16_t>(d, pl, scores, noise, indices, weights, ws, s);
+    return GCA_ERR_DTYPE;
+}
+
+// ------------------------------------------------------------------------------------ backward
+
+// Gradient of the retrieval weights w.r.t. the landmark embeddings, the selection held fixed:
+//   weights = softmax_k(scores[n, c, idx_k]),  scores = <lmk_q, lmk_k> / sqrt(hidden)
+//   ds_k = w_k (dw_k - sum_j w_j dw_j) / sqrt(hidden)        (slots of weight 0 -- masked ones -- get 0)
+//   dlmk_q[n, c] = sum_k ds_k lmk_k[n, idx_k]                 gather, one workgroup per row
+//   dlmk_k[n, e] = sum_{(c,k): idx = e} ds[n, c, k] lmk_q[n, c]   per landmark over its reference list
+// The lists are the ones the indexed attention backward uses (fixed order, no atomics).
+__global__ void __launch_bounds__(64)
+lmk_bwd_ds_kernel(lmk_desc d, int kk, const float* __restrict__ w, const float* __restrict__ dw, float* __restrict__ ds) {
+    const int64_t row = (int64_t)blockIdx.x * 64 + threadIdx.x;
+    if (row >= d.N * d.C) return;
+    float dot = 0.f;
+    for (int k = 0; k < kk; ++k) dot += w[row * kk + k] * dw[row * kk + k];
+    const float inv = 1.f / sqrtf(d.hidden_size);
+    for (int k = 0; k < kk; ++k) ds[row * kk + k] = w[row * kk + k] * (dw[row * kk + k] - dot) * inv;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+lmk_bwd_dq_kernel(lmk_desc d, int kk, const T* __restrict__ lk, const int64_t* __restrict__ idx,
+                  const float* __restrict__ ds, T* __restrict__ dlq) {
+    const int64_t row = blockIdx.x;
+    const int64_t n = row / d.C;
+    for (int i = threadIdx.x; i < d.Dm; i += 256) {
+        float acc = 0.f;
+        for (int k = 0; k < kk; ++k) {
+            const float g = ds[row * kk + k];
+            if (g != 0.f) acc = fmaf(g, to_f(lk[(n * d.E + clamp_idx(idx[row * kk + k], d.E)) * d.Dm + i]), acc);
+        }
+        dlq[row * d.Dm + i] = from_f<T>(acc);
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+lmk_bwd_dk_kernel(lmk_desc d, int kk, const T* __restrict__ lq, const float* __restrict__ ds, T* __restrict__ dlk,
+                  ListWs ws) {
+    const int64_t ce = blockIdx.x;                 // n * E + e
+    const int cnt = ws.count[ce], start = ws.start[ce];
+    for (int i = threadIdx.x; i < d.Dm; i += 256) {
+        float acc = 0.f;
+        for (int r = 0; r < cnt; ++r) {
+            const int ref = ws.refs[start + r];    // (n*C + c) * kk + k
+            acc = fmaf(ds[ref], to_f(lq[(int64_t)(ref / kk) * d.Dm + i]), acc);
+        }
+        dlk[ce * d.Dm + i] = from_f<T>(acc);
+    }
+}
+
+static Params lists_params(const lmk_desc& d, int kk) {
+    Params p = {};
+    p.Z = d.N * d.C; p.K = kk; p.N = d.N; p.C = d.E; p.zpn = d.C; p.indexed = 1;
+    p.Hkv = 1; p.K_CTX = 0; p.D = 0;       // no partial tiles
+    return p;
+}
+constexpr int LMK_SEG_MAX = 1 << 30;       // every list is walked whole
+
+size_t lmk_bwd_ws_bytes(const lmk_desc& d) {
+    const int kk = (int)((int64_t)d.topk < d.E ? d.topk : d.E);
+    const size_t dsb = ((size_t)d.N * d.C * kk * sizeof(float) + 255) / 256 * 256;
+    return dsb + list_ws_bytes(lists_params(d, kk), LMK_SEG_MAX);
+}
+
+template <typename T>
+static int launch_lmk_bwd_t(const lmk_desc& d, int kk, const void* lq, const void* lk, const int64_t* idx,
+                            const float* w, const float* dw, void* dlq, void* dlk, void* wsp, hipStream_t s) {
+    const int64_t R = d.N * d.C;
+    if (R > 0x7fffffffLL || d.N * d.E > 0x7fffffffLL) return GCA_ERR_SHAPE;
+    float* ds = (float*)wsp;
+    const size_t dsb = ((size_t)R * kk * sizeof(float) + 255) / 256 * 256;
+    const Params p = lists_params(d, kk);
+    const ListWs ws = list_carve(p, LMK_SEG_MAX, (char*)wsp + dsb);
+    hipLaunchKernelGGL(lmk_bwd_ds_kernel, dim3((unsigned)((R + 63) / 64)), dim3(64), 0, s, d, kk, w, dw, ds);
+    hipLaunchKernelGGL((lmk_bwd_dq_kernel<T>), dim3((unsigned)R), dim3(256), 0, s, d, kk, (const T*)lk, idx, ds, (T*)dlq);
+    if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
+    const int rc = list_build(p, LMK_SEG_MAX, idx, ws, s);
+    if (rc != GCA_OK) return rc;
+    hipLaunchKernelGGL((lmk_bwd_dk_kernel<T>), dim3((unsigned)(d.N * d.E)), dim3(256), 0, s, d, kk, (const T*)lq, ds, (T*)dlk, ws);
+    return hipGetLastError() == hipSuccess ? GCA_OK : GCA_ERR_LAUNCH;
+}
+
+int launch_lmk_bwd(const lmk_desc& d, const void* lq, const void* lk, const int64_t* idx, const float* w,
+                   const float* dw, void* dlq, void* dlk, void* wsp, size_t ws_bytes, hipStream_t s) {
+    const int kk = (int)((int64_t)d.topk < d.E ? d.topk : d.E);
+    if (wsp == nullptr || ws_bytes < lmk_bwd_ws_bytes(d)) return GCA_ERR_WORKSPACE;
+    if (d.dtype == GCA_F32) return launch_lmk_bwd_t<float>(d, kk, lq, lk, idx, w, dw, dlq, dlk, wsp, s);
+    if (d.dtype == GCA_BF16) return launch_lmk_bwd_t<bf16_t>(d, kk, lq, lk, idx, w, dw, dlq, dlk, wsp, s);
     return GCA_ERR_DTYPE;
 }
 

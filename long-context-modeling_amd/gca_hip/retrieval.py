@@ -60,11 +60,44 @@ def landmark_topk(scores, topk, causal=True, noise=None):
     return indices, weights
 
 
+class _Retrieve(torch.autograd.Function):
+    """Scoring + selection with a backward: the gradient of the weights flows to both landmark
+    embeddings (what autograd does through model/DRT.py:612 and :626-627); the selection is constant."""
+
+    @staticmethod
+    def forward(ctx, lmk_q, lmk_k, topk, hidden_size, causal, noise):
+        lmk_q, lmk_k = lmk_q.contiguous(), lmk_k.contiguous()
+        scores = landmark_scores(lmk_q, lmk_k, hidden_size, causal)
+        indices, weights = landmark_topk(scores, topk, causal, noise)
+        ctx.save_for_backward(lmk_q, lmk_k, indices, weights)
+        ctx.hidden, ctx.topk, ctx.causal = float(hidden_size), int(topk), bool(causal)
+        ctx.mark_non_differentiable(scores, indices)
+        return scores, indices, weights
+
+    @staticmethod
+    def backward(ctx, _dscores, _dindices, dweights):
+        lmk_q, lmk_k, indices, weights = ctx.saved_tensors
+        N, C, Dm = lmk_q.shape
+        E = lmk_k.shape[1]
+        dweights = dweights.contiguous().float()
+        dlq, dlk = torch.empty_like(lmk_q), torch.empty_like(lmk_k)
+        desc = _lmk_desc(lmk_q.dtype, ctx.topk, N, C, E, Dm, ctx.causal, ctx.hidden)
+        with torch.cuda.device(lmk_q.device):
+            L = _lib.lib()
+            nbytes = L.lmk_weights_bwd_workspace_bytes(ctypes.byref(desc))
+            ws = torch.empty(nbytes // 4 + 1, device=lmk_q.device, dtype=torch.float32)
+            rc = L.lmk_weights_bwd(ctypes.byref(desc), _ptr(lmk_q), _ptr(lmk_k), _ptr(indices), _ptr(weights),
+                                   _ptr(dweights), _ptr(dlq), _ptr(dlk), _ptr(ws), nbytes, _stream(lmk_q.device))
+        _lib.check(rc, "lmk_weights_bwd")
+        return dlq, dlk, None, None, None, None
+
+
 def landmark_retrieve(lmk_q, lmk_k, topk, hidden_size=None, causal=True, noise=None):
-    """Scoring + selection in one call.  Returns (scores, indices, weights)."""
-    scores = landmark_scores(lmk_q, lmk_k, hidden_size, causal)
-    indices, weights = landmark_topk(scores, topk, causal, noise)
-    return scores, indices, weights
+    """Scoring + selection in one call.  Returns (scores, indices, weights); ``weights`` carries the
+    gradient to ``lmk_q`` and ``lmk_k``."""
+    assert lmk_q.is_cuda and lmk_q.dim() == 3 and lmk_k.dim() == 3
+    hidden_size = lmk_q.shape[-1] if hidden_size is None else hidden_size
+    return _Retrieve.apply(lmk_q, lmk_k, topk, hidden_size, causal, noise)
 
 
 def gather_chunks(chunk_k, chunk_v, indices, weights, num_kv_heads):
