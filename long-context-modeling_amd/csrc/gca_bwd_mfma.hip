@@ -42,15 +42,15 @@ static const int SEG_MAX = seg_max_from_env();
 // ------------------------------------------------------------------------------------------- dq
 
 template <int D, int GS, bool INDEXED>
-__global__ void __launch_bounds__(128 * GS) __attribute__((amdgpu_waves_per_eu(D == 64 ? 2 : 1)))
+__global__ void __launch_bounds__(128 * GS) __attribute__((amdgpu_waves_per_eu(D == 64 ? 3 : 1)))
 gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
                        const uint16_t* __restrict__ v, const int64_t* __restrict__ indices,
                        const void* __restrict__ w, int w_is_bf16, const uint16_t* __restrict__ dout,
                        const float* __restrict__ lse, uint16_t* __restrict__ dq, float* __restrict__ delta) {
     constexpr int NT = 128 * GS;
     constexpr int KS = D / 16, DB = D / 32;
-    constexpr int RB = D * 2, TILE = 64 * RB, BUF = 2 * TILE;
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * BUF];
+    constexpr int RB = D * 2, TILE = 64 * RB;
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[3 * TILE];   // two K tiles (K is read in both phases), one V tile
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -90,7 +90,7 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
     {
         int64_t rs;
         loader.issue(chunk_base_n(p, k, indices, nseq, z, hk, 0, rs), smem);
-        loader.issue(chunk_base_n(p, v, indices, nseq, z, hk, 0, rs), smem + TILE);
+        loader.issue(chunk_base_n(p, v, indices, nseq, z, hk, 0, rs), smem + 2 * TILE);
     }
     wait_async_tiles();
     __syncthreads();
@@ -101,12 +101,11 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
 
     for (int j = 0; j < p.K; ++j) {
         const int buf = j & 1;
-        if (j + 1 < p.K) {
-            // the other buffer was last read in iteration j-1, which every wavefront has left
+        const bool more = j + 1 < p.K;
+        if (more) {
+            // the other K buffer was last read in iteration j-1, which every wavefront has left
             int64_t rs;
-            unsigned char* nb = smem + (buf ^ 1) * BUF;
-            loader.issue(chunk_base_n(p, k, indices, nseq, z, hk, j + 1, rs), nb);
-            loader.issue(chunk_base_n(p, v, indices, nseq, z, hk, j + 1, rs), nb + TILE);
+            loader.issue(chunk_base_n(p, k, indices, nseq, z, hk, j + 1, rs), smem + (buf ^ 1) * TILE);
         }
         // mult = w_j * sm_scale multiplies dS; it rides in the exponent: Pm = mult * P = exp2(c S - lse + log2 mult).
         // A slot of weight 0 gives dS = 0: its P is left unscaled (delta is still needed) and the dQ product skipped.
@@ -114,8 +113,8 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
         const bool live = mult > 0.f;
         const float eoff = lse[lrow + (int64_t)j * p.Q_CTX] - (live ? __builtin_amdgcn_logf(mult) : 0.f);
         const float dscale = live ? 1.f / mult : 1.f;
-        const unsigned char* kb = smem + buf * BUF;
-        const unsigned char* vb = kb + TILE;
+        const unsigned char* kb = smem + buf * TILE;
+        const unsigned char* vb = smem + 2 * TILE;
 
         f32x16 st[2], dpt[2];
 #pragma unroll
@@ -129,6 +128,12 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
                 st[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(kb + po), qB[ks], st[t], 0, 0, 0);
                 dpt[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(vb + po), doB[ks], dpt[t], 0, 0, 0);
             }
+        }
+        // every wavefront is done with the V tile (only dP^T reads it): refill it for chunk j+1
+        __syncthreads();
+        if (more) {
+            int64_t rs;
+            loader.issue(chunk_base_n(p, v, indices, nseq, z, hk, j + 1, rs), smem + 2 * TILE);
         }
         float dsum = 0.f;
 #pragma unroll

@@ -26,15 +26,15 @@
 namespace gca {
 
 template <int D, int GS, bool INDEXED>
-__global__ void __launch_bounds__(128 * GS) __attribute__((amdgpu_waves_per_eu(2)))
+__global__ void __launch_bounds__(128 * GS) __attribute__((amdgpu_waves_per_eu(D == 64 ? 4 : 2)))
 gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
                     const uint16_t* __restrict__ v, const int64_t* __restrict__ indices,
                     const void* __restrict__ w, int w_is_bf16, uint16_t* __restrict__ o, float* __restrict__ lse) {
     constexpr int NT = 128 * GS;
     constexpr int KS = D / 16;                 // reduction steps of Q.K^T
     constexpr int DB = D / 32;                 // 32-wide dim blocks of O
-    constexpr int RB = D * 2, TILE = 64 * RB, BUF = 2 * TILE;   // K tile then V tile
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * BUF];
+    constexpr int RB = D * 2, TILE = 64 * RB;
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * TILE];   // one K tile, one V tile
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -72,30 +72,25 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
 
     const float c = p.sm_scale * LOG2E;
 
-    const TileLoader<D, NT> loader(tid, INDEXED ? p.Hkv * D : D);
+    // One K tile and one V tile in LDS.  Per chunk: S phase reads K; barrier; the K tile is refilled with
+    // chunk j+1 while the softmax runs; V (issued one phase earlier) is waited for right before P.V; after
+    // P.V the V tile is refilled.  Loads retire in order, so "all but the newest NI" isolates the older copy.
+    using Loader = TileLoader<D, NT>;
+    const Loader loader(tid, INDEXED ? p.Hkv * D : D);
     {
         int64_t rs;
         loader.issue(chunk_base_n(p, k, indices, nseq, z, hk, 0, rs), smem);
         loader.issue(chunk_base_n(p, v, indices, nseq, z, hk, 0, rs), smem + TILE);
     }
-    wait_async_tiles();
+    wait_async_tiles_but<Loader::NI>();     // K of chunk 0 has landed, V may still be in flight
     __syncthreads();
 
     const TrLane tr(lane);
     const int fsw = swz(n);
 
     for (int j = 0; j < p.K; ++j) {
-        const int buf = j & 1;
-        if (j + 1 < p.K) {
-            // the other buffer was last read in iteration j-1, which every wavefront has left
-            int64_t rs;
-            unsigned char* nb = smem + (buf ^ 1) * BUF;
-            loader.issue(chunk_base_n(p, k, indices, nseq, z, hk, j + 1, rs), nb);
-            loader.issue(chunk_base_n(p, v, indices, nseq, z, hk, j + 1, rs), nb + TILE);
-        }
-
-        const unsigned char* kb = smem + buf * BUF;
-        const unsigned char* vb = kb + TILE;
+        const unsigned char* kb = smem;
+        const unsigned char* vb = smem + TILE;
 
         // ---- S^T = K Q^T : two 32-key tiles, keys in registers, query n in the lane
         f32x16 st[2];
@@ -109,6 +104,14 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
                 const bf16x8 a = lds_read_b128(kb + rowoff + (((2 * ks + h) ^ fsw) << 4));
                 st[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qB[ks], st[t], 0, 0, 0);
             }
+        }
+
+        // every wavefront is done with the K tile: refill it with chunk j+1 while the softmax and P.V run
+        __syncthreads();
+        const bool more = j + 1 < p.K;
+        if (more) {
+            int64_t rs;
+            loader.issue(chunk_base_n(p, k, indices, nseq, z, hk, j + 1, rs), smem);
         }
 
         // ---- softmax over the 64 keys of this chunk for query n
@@ -144,7 +147,9 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
 #pragma unroll
             for (int s = 0; s < 8; ++s) pA[t4][s] = (__bf16)(st[t4 >> 1][8 * (t4 & 1) + s] * inv);
 
-        // ---- O += P~ V
+        // ---- O += P~ V   (this chunk's V copy is older than the K refill just issued)
+        if (more) wait_async_tiles_but<Loader::NI>(); else wait_async_tiles();
+        __syncthreads();
 #pragma unroll
         for (int t4 = 0; t4 < 4; ++t4) {
 #pragma unroll
@@ -155,8 +160,13 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
             }
         }
 
-        wait_async_tiles();
-        __syncthreads();
+        // the K refill has landed and every wavefront is done with the V tile: refill V for chunk j+1
+        if (more) {
+            wait_async_tiles();
+            __syncthreads();
+            int64_t rs;
+            loader.issue(chunk_base_n(p, v, indices, nseq, z, hk, j + 1, rs), smem + TILE);
+        }
     }
 
     // ---- store O: register r of block db is row 8*(r/4) + 4*h + r%4, column 32*db + n

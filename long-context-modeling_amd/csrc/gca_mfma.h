@@ -107,6 +107,13 @@ __device__ __forceinline__ void async_row64(const float* src, float* lds_dst, in
 
 // all outstanding global_load_lds of this wavefront have landed (vmcnt = 0; other counters untouched)
 __device__ __forceinline__ void wait_async_tiles() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+// all but the NEWEST most recent vector-memory operations of this wavefront have completed (loads
+// retire in order, so everything issued before the last NEWEST instructions has landed); NEWEST <= 15
+template <int NEWEST>
+__device__ __forceinline__ void wait_async_tiles_but() {
+    static_assert(NEWEST >= 0 && NEWEST <= 15, "vmcnt immediate");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | NEWEST);
+}
 
 // XCD-aware work order.  The hardware deals workgroups round-robin to the 8 XCDs (workgroup i runs
 // on XCD i % 8), each with its own L2.  Work items are numbered so that items sharing data are
