@@ -26,6 +26,9 @@ for _p in (ROOT, os.path.join(ROOT, "long-context-modeling_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the three main kernels at config 2, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# scaled by the same counters' readings for a 1 GiB device copy (profiles/gca_step_cfg2_bf16.txt)
+MEASURED_TRAFFIC_GB = {"gca_fwd_mfma_kernel": 1.169, "gca_bwd_dq_mfma_kernel": 1.609, "gca_bwd_dkdv2_mfma_kernel": 1.853}
 
 
 def log(*a):
@@ -99,7 +102,9 @@ def kernel_times(torch, q, ck, cv, idx, w, do, sm_scale, sm_n, iters):
     times = {
         "gca_fwd_mfma_kernel": event_time(torch, fwd, iters),
         "gca_bwd_dq_mfma_kernel": event_time(torch, bwd(1), iters),
-        "gca_bwd_dkdv_mfma_kernel(+lists)": event_time(torch, bwd(2), iters),
+        "gca_list_build(3 launches)": event_time(torch, bwd(8), iters),
+        "gca_bwd_dkdv2_mfma_kernel": event_time(torch, bwd(2), iters),
+        "gca_bwd_dkdv_reduce_kernel": event_time(torch, bwd(16), iters),
         "gca_bwd_dw_kernel": event_time(torch, bwd(4), iters),
     }
     return times
@@ -293,12 +298,15 @@ def main():
     b_fwd = 2 * H * d * e + 2 * K * H * d * e + 4 * H * K
     b_dq = 2 * H * d * e + 4 * H * K + 2 * K * H * d * e + H * d * e          # q, dO, lse, gather, dq
     b_dkdv = 2 * K * H * d * 4                                                # fp32 dK/dV accumulation
-    model = {"gca_fwd_mfma_kernel": b_fwd, "gca_bwd_dq_mfma_kernel": b_dq, "gca_bwd_dkdv_mfma_kernel(+lists)": b_dkdv}
+    model = {"gca_fwd_mfma_kernel": b_fwd, "gca_bwd_dq_mfma_kernel": b_dq, "gca_bwd_dkdv2_mfma_kernel": b_dkdv}
     dom = max(model, key=lambda k_: kt[k_])
     achieved = model[dom] * tokens / (kt[dom] * 1e-3) / 1e9
     step_bytes = (b_fwd + b_dq + b_dkdv) * tokens
     roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": round(MEASURED_TRAFFIC_GB[dom] / (kt[dom] * 1e-3), 1),
+                "traffic_GB_per_launch": MEASURED_TRAFFIC_GB[dom],
+                "algorithmic_GB_per_launch": round(model[dom] * tokens / 1e9, 3),
                 "kernel_ms": {k_: round(v, 4) for k_, v in kt.items()},
                 "step_algorithmic_GB": round(step_bytes / 1e9, 3),
                 "step_frac_of_hbm_roofline": round(step_bytes / dt / 1e9 / HBM_PEAK_GBS, 4)}

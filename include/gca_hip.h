@@ -58,8 +58,10 @@ enum gca_path { GCA_PATH_AUTO = 0, GCA_PATH_GENERIC = 1, GCA_PATH_MFMA = 2 };
  * later stage alone needs the buffers an earlier stage fills (delta in the workspace). */
 enum gca_stage {
     GCA_STAGE_DQ = 1,      /* dq and the per-chunk row sums delta */
-    GCA_STAGE_DKDV = 2,    /* reference lists (indexed form) and dk, dv */
-    GCA_STAGE_DW = 4       /* dw from delta */
+    GCA_STAGE_DKDV = 2,    /* the dk/dv kernel (needs delta; indexed form: needs the lists) */
+    GCA_STAGE_DW = 4,      /* dw from delta */
+    GCA_STAGE_LISTS = 8,   /* indexed form: build the reference lists in the workspace */
+    GCA_STAGE_REDUCE = 16  /* indexed form: add up the partial tiles of chunks with long lists */
 };
 
 typedef struct gca_desc {

@@ -270,17 +270,17 @@ static int launch_d(const Params& p, const void* q, const void* k, const void* v
         hipLaunchKernelGGL((gca_bwd_dq_generic_kernel<T, WT, D>), dim3((unsigned)b1), dim3(256), 0, s, p,
                            (const T*)q, (const T*)k, (const T*)v, idx, (const WT*)w, (const T*)dout, lse, (T*)dq, delta);
     if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
-    if (!(p.stages & GCA_STAGE_DKDV)) return (p.stages & GCA_STAGE_DW) ? launch_dw(p, delta, dw, s) : GCA_OK;
     ListWs ws = {};
     if (p.indexed) {
         // every chunk's list is walked whole by one workgroup here: no segments, no partial slots
         ws = list_carve(p, GENERIC_SEG_MAX, (char*)delta + delta_bytes(p));
-        const int rc = list_build(p, GENERIC_SEG_MAX, idx, ws, s);
+        const int rc = (p.stages & GCA_STAGE_LISTS) ? list_build(p, GENERIC_SEG_MAX, idx, ws, s) : GCA_OK;
         if (rc != GCA_OK) return rc;
+        if (p.stages & GCA_STAGE_DKDV)
         hipLaunchKernelGGL((gca_bwd_dkdv_generic_kernel<T, WT, D, true>), dim3((unsigned)b2), dim3(256), 0, s, p,
                            (const T*)q, (const T*)k, (const T*)v, idx, (const WT*)w, (const T*)dout, lse, delta,
                            (T*)dk, (T*)dv, ws);
-    } else {
+    } else if (p.stages & GCA_STAGE_DKDV) {
         hipLaunchKernelGGL((gca_bwd_dkdv_generic_kernel<T, WT, D, false>), dim3((unsigned)b2), dim3(256), 0, s, p,
                            (const T*)q, (const T*)k, (const T*)v, idx, (const WT*)w, (const T*)dout, lse, delta,
                            (T*)dk, (T*)dv, ws);

@@ -672,19 +672,19 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
         else rc = launch_dq_gs<D, 1>(p, q, k, v, idx, w, wb, dout, lse, dq, delta, s);
         if (rc != GCA_OK) return rc;
     }
-    if (!(p.stages & GCA_STAGE_DKDV)) return (p.stages & GCA_STAGE_DW) ? launch_dw(p, delta, dw, s) : GCA_OK;
 
     ListWs ws = {};
     const int seg_per0 = 0;
     if (p.indexed) {
         // the list workspace follows delta
         ws = list_carve(p, SEG_MAX, (char*)delta + delta_bytes(p));
-        if ((rc = list_build(p, SEG_MAX, idx, ws, s)) != GCA_OK) return rc;
+        if ((p.stages & GCA_STAGE_LISTS) && (rc = list_build(p, SEG_MAX, idx, ws, s)) != GCA_OK) return rc;
         // segment slots per sequence: every chunk has one segment, plus one per SEG_MAX references
         const int seg_per = (int)(p.C + (p.zpn * p.K + SEG_MAX - 1) / SEG_MAX);
         const int64_t blocks = (p.N * p.Hkv + NUM_XCD - 1) / NUM_XCD * NUM_XCD * seg_per;
         if (blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
-        if (D == 64)
+        if (!(p.stages & GCA_STAGE_DKDV)) {
+        } else if (D == 64)
             hipLaunchKernelGGL((gca_bwd_dkdv2_mfma_kernel<D, true>), dim3((unsigned)blocks), dim3(128), 0, s, p,
                                (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
                                delta, dk, dv, ws, seg_per);
@@ -692,12 +692,14 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
             hipLaunchKernelGGL((gca_bwd_dkdv_mfma_kernel<D, true>), dim3((unsigned)blocks), dim3(256), 0, s, p,
                                (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
                                delta, dk, dv, ws, seg_per);
-        hipLaunchKernelGGL((gca_bwd_dkdv_reduce_kernel<D>), dim3((unsigned)(p.N * p.C * p.Hkv)), dim3(256), 0, s, p, SEG_MAX,
-                           (uint16_t*)dk, (uint16_t*)dv, ws);
+        if (p.stages & GCA_STAGE_REDUCE)
+            hipLaunchKernelGGL((gca_bwd_dkdv_reduce_kernel<D>), dim3((unsigned)(p.N * p.C * p.Hkv)), dim3(256), 0, s, p, SEG_MAX,
+                               (uint16_t*)dk, (uint16_t*)dv, ws);
     } else {
         const int64_t blocks = p.Z * p.Hkv * p.K;
         if (blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
-        if (D == 64)
+        if (!(p.stages & GCA_STAGE_DKDV)) {
+        } else if (D == 64)
             hipLaunchKernelGGL((gca_bwd_dkdv2_mfma_kernel<D, false>), dim3((unsigned)blocks), dim3(128), 0, s, p,
                                (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
                                delta, dk, dv, ws, seg_per0);

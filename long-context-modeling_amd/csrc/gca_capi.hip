@@ -14,7 +14,7 @@ int check_desc(const gca_desc* d, bool indexed) {
     if (d->D != 16 && d->D != 32 && d->D != 64 && d->D != 128 && d->D != 256) return GCA_ERR_SHAPE;
     if (!(d->sm_n >= 0.f)) return GCA_ERR_SHAPE;
     if (d->path != GCA_PATH_AUTO && d->path != GCA_PATH_GENERIC && d->path != GCA_PATH_MFMA) return GCA_ERR_SHAPE;
-    if (d->stages < 0 || d->stages > 7) return GCA_ERR_SHAPE;
+    if (d->stages < 0 || d->stages > 31) return GCA_ERR_SHAPE;
     if (indexed) {
         if (d->N <= 0 || d->C <= 0 || d->Z % d->N != 0) return GCA_ERR_SHAPE;
     }

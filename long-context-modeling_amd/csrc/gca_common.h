@@ -48,7 +48,7 @@ inline Params make_params(const gca_desc& d, bool indexed) {
     p.N = indexed ? d.N : 1; p.C = indexed ? d.C : 1;
     p.zpn = indexed ? d.Z / d.N : d.Z;
     p.indexed = indexed ? 1 : 0;
-    p.stages = d.stages == 0 ? 7 : d.stages;
+    p.stages = d.stages == 0 ? 31 : d.stages;
     return p;
 }
 
