@@ -6,10 +6,13 @@
 //               16-byte loads, wavefront reduction.  "mfma": many query rows in bf16 (training/prefill): 64x128 score blocks
 //               on the matrix cores, operands through swizzled LDS tiles.  "tile": the fp32 path and
 //               odd widths: 32x32 output tiles on the vector ALUs.  Fully masked blocks are only filled.
-//   lmk_topk    bitonic top-k in LDS over 64-bit keys (order-preserving image of the float in
-//               the high half, inverted index in the low half), so "higher value first, then
-//               lower index" is one unsigned compare and the result is unique.  Long rows are
-//               cut into segments (one workgroup each) whose winners a second launch merges.
+//   lmk_topk    bitonic top-k over 64-bit keys (order-preserving image of the float in the high
+//               half, inverted index in the low half), so "higher value first, then lower index"
+//               is one unsigned compare and the result is unique.  k <= 32: every thread sorts its
+//               own keys in registers, butterfly merges inside the wavefront need no barrier, the
+//               four wavefronts meet through LDS.  Larger k: the whole network runs on LDS tiles.
+//               Long rows are cut into segments (one workgroup each) whose winners a second
+//               launch merges.
 #include "gca_mfma.h"
 #include "gca_lists.h"
 
@@ -427,6 +430,105 @@ __device__ void block_topk(uint64_t* keys, int kp, int tid) {
     __syncthreads();
 }
 
+// ---- register / shuffle tournament for kp <= 32 --------------------------------------------------
+// Each thread owns KP keys, sorted descending in registers.  merge_from() replaces them by the KP
+// largest of (mine, other's): with both lists descending, max(mine[i], other[KP-1-i]) is the half-cleaner
+// of a bitonic sequence, and log2(KP) compare-exchange stages sort the result again.  Six butterfly
+// levels (lane ^ 1, 2, ..., 32) leave the wavefront's winners in every lane with no barrier; the four
+// wavefronts then meet through LDS.  All keys are distinct (the index is part of the key) or 0 (padding).
+__device__ __forceinline__ uint64_t shfl_xor_key(uint64_t v, int mask) {
+    const uint32_t lo = __shfl_xor((uint32_t)v, mask), hi = __shfl_xor((uint32_t)(v >> 32), mask);
+    return ((uint64_t)hi << 32) | lo;
+}
+__device__ __forceinline__ uint32_t shfl_xor_key(uint32_t v, int mask) { return __shfl_xor(v, mask); }
+
+template <typename KT, int KP>
+__device__ __forceinline__ void sort_desc_regs(KT (&a)[KP]) {
+#pragma unroll
+    for (int size = 2; size <= KP; size <<= 1)
+#pragma unroll
+        for (int stride = size >> 1; stride > 0; stride >>= 1)
+#pragma unroll
+            for (int i = 0; i < KP; ++i) {
+                const int l = i ^ stride;
+                if (l > i) {
+                    // sub-lists alternate direction until the last pass, which sorts the whole list descending
+                    const bool up = ((i & size) != 0) && size != KP;
+                    const KT x = a[i], y = a[l];
+                    const bool sw = up ? (x > y) : (x < y);
+                    a[i] = sw ? y : x;
+                    a[l] = sw ? x : y;
+                }
+            }
+}
+
+template <typename KT, int KP>
+__device__ __forceinline__ void merge_from(KT (&a)[KP], const KT (&b)[KP]) {
+#pragma unroll
+    for (int i = 0; i < KP; ++i) a[i] = a[i] > b[KP - 1 - i] ? a[i] : b[KP - 1 - i];
+#pragma unroll
+    for (int stride = KP >> 1; stride > 0; stride >>= 1)
+#pragma unroll
+        for (int i = 0; i < KP; ++i) {
+            const int l = i ^ stride;
+            if (l > i) {
+                const KT x = a[i], y = a[l];
+                const bool sw = x < y;
+                a[i] = sw ? y : x;
+                a[l] = sw ? x : y;
+            }
+        }
+}
+
+// Every thread passes its KP sorted keys; on return thread 0 holds the KP largest of the workgroup,
+// sorted descending.  xch: 4 * KP keys of LDS.  All TOPK_THREADS threads must call it.
+template <typename KT, int KP>
+__device__ __forceinline__ void block_tournament(KT (&a)[KP], KT* xch, int tid) {
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) {
+        KT b[KP];
+#pragma unroll
+        for (int i = 0; i < KP; ++i) b[i] = shfl_xor_key(a[i], m);
+        merge_from<KT, KP>(a, b);
+    }
+    const int lane = tid & 63, wave = tid >> 6;
+    __syncthreads();                       // xch may still be read by the previous round
+    if (lane == 0)
+#pragma unroll
+        for (int i = 0; i < KP; ++i) xch[wave * KP + i] = a[i];
+    __syncthreads();
+    if (tid == 0)
+#pragma unroll
+        for (int wv = 1; wv < TOPK_THREADS / 64; ++wv) {
+            KT b[KP];
+#pragma unroll
+            for (int i = 0; i < KP; ++i) b[i] = xch[wv * KP + i];
+            merge_from<KT, KP>(a, b);
+        }
+}
+
+// Keys used inside a segment.  float scores need the full 64-bit key.  bf16 scores have 16 significant
+// bits, so (16-bit order-preserving value, 16-bit inverted offset in the segment) fits 32 bits and the
+// compare/select chains are half as long; segments of bf16 rows are therefore at most 65536 long.
+template <typename T> struct SegKey;
+template <> struct SegKey<float> {
+    typedef uint64_t type;
+    static __device__ __forceinline__ uint64_t make(float v, int64_t e, int64_t) { return make_key(v, (uint32_t)e); }
+    static __device__ __forceinline__ uint64_t global(uint64_t k, int64_t) { return k; }
+};
+template <> struct SegKey<bf16_t> {
+    typedef uint32_t type;
+    static __device__ __forceinline__ uint32_t make(float v, int64_t e, int64_t lo) {
+        return (sortable_bits(v) & 0xffff0000u) | (0xffffu - (uint32_t)(e - lo));    // v is a bf16 value: low bits carry nothing
+    }
+    static __device__ __forceinline__ uint64_t global(uint32_t k, int64_t lo) {
+        if (k == 0) return 0;
+        const uint32_t e = (uint32_t)lo + (0xffffu - (k & 0xffffu));
+        return ((uint64_t)(k | 0xffffu) << 32) | (uint64_t)(0xffffffffu - e);
+    }
+};
+constexpr int64_t SEG_MAX_BF16 = 65536;
+
 template <typename T>
 __device__ __forceinline__ float round_like(float x);
 template <> __device__ __forceinline__ float round_like<float>(float x) { return x; }
@@ -529,15 +631,109 @@ lmk_topk_merge_kernel(lmk_desc d, int kk, int kp, int nseg, int64_t row0, const 
     emit_row<T>(d, keys, kk, row, limit, scores, indices, weights, sval, tid);
 }
 
+// Tournament version of the two kernels above for kp <= 32.  A tile is TOPK_THREADS * KP candidates.
+template <typename T, int KP>
+__global__ void __launch_bounds__(TOPK_THREADS)
+lmk_topk_reg_kernel(lmk_desc d, int kk, int nseg, int64_t seg_len, int64_t row0, const T* __restrict__ scores,
+                    const T* __restrict__ noise, int64_t* __restrict__ indices, float* __restrict__ weights,
+                    uint64_t* __restrict__ ws) {
+    typedef typename SegKey<T>::type KT;
+    __shared__ KT xch[(TOPK_THREADS / 64) * KP];
+    __shared__ uint64_t win[KP];
+    __shared__ float sval[TOPK_MAX_KP];
+    const int tid = threadIdx.x;
+    const int seg = blockIdx.x;
+    const int64_t row = row0 + blockIdx.y;
+    const int64_t c = row % d.C;
+    const int64_t limit = d.causal ? (d.E - d.C + c) : d.E;
+    const int64_t scan_end = min(d.E, max(limit, (int64_t)kk));
+    const int64_t lo = (int64_t)seg * seg_len;
+    const int64_t hi = min(lo + seg_len, scan_end);
+    KT best[KP];
+#pragma unroll
+    for (int i = 0; i < KP; ++i) best[i] = 0;
+    for (int64_t pos = lo; pos < hi || pos == lo; pos += (int64_t)TOPK_THREADS * KP) {
+        KT a[KP];
+#pragma unroll
+        for (int i = 0; i < KP; ++i) {
+            const int64_t e = pos + (int64_t)i * TOPK_THREADS + tid;       // coalesced across the workgroup
+            KT key = 0;
+            if (e < hi) {
+                float sv = to_f(scores[row * d.E + e]);
+                if (noise != nullptr) sv = round_like<T>(sv + to_f(noise[row * d.E + e]));
+                if (d.causal && !(e < limit)) sv = -INFINITY;
+                key = SegKey<T>::make(sv, e, lo);
+            }
+            a[i] = key;
+        }
+        sort_desc_regs<KT, KP>(a);
+        block_tournament<KT, KP>(a, xch, tid);
+        if (tid == 0) merge_from<KT, KP>(best, a);
+    }
+    if (tid == 0)
+#pragma unroll
+        for (int i = 0; i < KP; ++i) win[i] = SegKey<T>::global(best[i], lo);
+    __syncthreads();
+    if (nseg == 1) {
+        emit_row<T>(d, win, kk, row, limit, scores, indices, weights, sval, tid);
+    } else if (tid < KP) {
+        ws[(row * nseg + seg) * KP + tid] = win[tid];
+    }
+}
+
+template <typename T, int KP>
+__global__ void __launch_bounds__(TOPK_THREADS)
+lmk_topk_reg_merge_kernel(lmk_desc d, int kk, int nseg, int64_t row0, const T* __restrict__ scores,
+                          int64_t* __restrict__ indices, float* __restrict__ weights, const uint64_t* __restrict__ ws) {
+    __shared__ uint64_t xch[(TOPK_THREADS / 64) * KP];
+    __shared__ uint64_t win[KP];
+    __shared__ float sval[TOPK_MAX_KP];
+    const int tid = threadIdx.x;
+    const int64_t row = row0 + blockIdx.x;
+    const int64_t c = row % d.C;
+    const int64_t limit = d.causal ? (d.E - d.C + c) : d.E;
+    // each segment's KP winners are already sorted descending: a thread takes whole segments
+    uint64_t best[KP];
+#pragma unroll
+    for (int i = 0; i < KP; ++i) best[i] = 0;
+    for (int sg = tid; sg < nseg; sg += TOPK_THREADS) {
+        uint64_t b[KP];
+#pragma unroll
+        for (int i = 0; i < KP; ++i) b[i] = ws[(row * nseg + sg) * KP + i];
+        merge_from<uint64_t, KP>(best, b);
+    }
+    block_tournament<uint64_t, KP>(best, xch, tid);
+    if (tid == 0)
+#pragma unroll
+        for (int i = 0; i < KP; ++i) win[i] = best[i];
+    __syncthreads();
+    emit_row<T>(d, win, kk, row, limit, scores, indices, weights, sval, tid);
+}
+
 static int next_pow2(int x) { int p = 1; while (p < x) p <<= 1; return p; }
 
 struct TopkPlan { int kk, kp, nseg; int64_t seg_len; };
+
+constexpr int TOPK_REG_MAX_KP = 32;     // largest kp the tournament kernels are built for
 
 static TopkPlan plan_topk(const lmk_desc& d) {
     TopkPlan pl;
     pl.kk = (int)((int64_t)d.topk < d.E ? d.topk : d.E);
     pl.kp = next_pow2(pl.kk);
     const int64_t R = d.N * d.C;
+    if (pl.kp <= TOPK_REG_MAX_KP) {
+        // tournament kernels: a segment is a whole number of tiles of TOPK_THREADS * kp candidates
+        const int64_t tile = (int64_t)TOPK_THREADS * pl.kp;
+        const int64_t tiles = (d.E + tile - 1) / tile;
+        int64_t want = (2048 + R - 1) / R;
+        if (want < 1) want = 1;
+        if (want > tiles) want = tiles;
+        if (want > 4096) want = 4096;
+        pl.seg_len = ((d.E + want - 1) / want + tile - 1) / tile * tile;
+        if (d.dtype == GCA_BF16 && pl.seg_len > SEG_MAX_BF16) pl.seg_len = SEG_MAX_BF16 / tile * tile;   // 32-bit segment keys
+        pl.nseg = (int)((d.E + pl.seg_len - 1) / pl.seg_len);
+        return pl;
+    }
     const int64_t tiles = (d.E + TOPK_TILE - 1) / TOPK_TILE;
     int64_t want = (2048 + R - 1) / R;          // aim at >= 2048 workgroups
     if (want < 1) want = 1;
@@ -554,9 +750,36 @@ size_t lmk_topk_ws_bytes(const lmk_desc& d) {
     return pl.nseg > 1 ? (size_t)(d.N * d.C) * pl.nseg * pl.kp * sizeof(uint64_t) : 0;
 }
 
+template <typename T, int KP>
+static int launch_topk_reg(const lmk_desc& d, const TopkPlan& pl, const void* scores, const void* noise,
+                           int64_t* indices, float* weights, void* ws, hipStream_t s) {
+    const int64_t R = d.N * d.C;
+    const int64_t slab = 65535;
+    for (int64_t r0 = 0; r0 < R; r0 += slab) {
+        const int64_t rows = (R - r0) < slab ? (R - r0) : slab;
+        hipLaunchKernelGGL((lmk_topk_reg_kernel<T, KP>), dim3((unsigned)pl.nseg, (unsigned)rows), dim3(TOPK_THREADS), 0, s, d,
+                           pl.kk, pl.nseg, pl.seg_len, r0, (const T*)scores, (const T*)noise, indices, weights, (uint64_t*)ws);
+        if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
+        if (pl.nseg > 1) {
+            hipLaunchKernelGGL((lmk_topk_reg_merge_kernel<T, KP>), dim3((unsigned)rows), dim3(TOPK_THREADS), 0, s, d, pl.kk,
+                               pl.nseg, r0, (const T*)scores, indices, weights, (const uint64_t*)ws);
+            if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
+        }
+    }
+    return GCA_OK;
+}
+
 template <typename T>
 static int launch_topk_t(const lmk_desc& d, const TopkPlan& pl, const void* scores, const void* noise,
                          int64_t* indices, float* weights, void* ws, hipStream_t s) {
+    switch (pl.kp) {
+        case 1: return launch_topk_reg<T, 1>(d, pl, scores, noise, indices, weights, ws, s);
+        case 2: return launch_topk_reg<T, 2>(d, pl, scores, noise, indices, weights, ws, s);
+        case 4: return launch_topk_reg<T, 4>(d, pl, scores, noise, indices, weights, ws, s);
+        case 8: return launch_topk_reg<T, 8>(d, pl, scores, noise, indices, weights, ws, s);
+        case 16: return launch_topk_reg<T, 16>(d, pl, scores, noise, indices, weights, ws, s);
+        case 32: return launch_topk_reg<T, 32>(d, pl, scores, noise, indices, weights, ws, s);
+    }
     // rows go in grid.y (at most 65535 per launch); rows are independent, so long inputs
     // are cut into slabs and each launch is told its first row
     const int64_t R = d.N * d.C;
