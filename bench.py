@@ -27,7 +27,7 @@ for _p in (ROOT, os.path.join(ROOT, "long-context-modeling_amd")):
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the three main kernels at config 2, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# scaled by the same counters' readings for a 1 GiB device copy (profiles/gca_step_cfg2_bf16.txt)
+# scaled by the same counters' readings for a 1 GiB device copy (summary kept under profiles/)
 MEASURED_TRAFFIC_GB = {"gca_fwd_mfma_kernel": 1.169, "gca_bwd_dq_mfma_kernel": 1.609, "gca_bwd_dkdv2_mfma_kernel": 1.853}
 
 
@@ -244,7 +244,7 @@ def main():
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (sharding is described in DESIGN.md)")
+        sys.exit("bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path is built)")
 
     import torch
     if not torch.cuda.is_available():

@@ -5,10 +5,12 @@
 // Work split.  A workgroup owns one (z, kv head, slice of GS query heads of the group, 64-row
 // query tile) and walks the K retrieved chunks.  It has 2*GS wavefronts; wavefront w owns the
 // 32 query rows qb = w % 2 of query head w / 2.  Each retrieved chunk's K and V tiles
-// (64 x D bf16 each) are read from HBM once per workgroup with 16-byte coalesced loads,
-// staged in LDS (double buffered: the asynchronous loads of chunk j+1 are issued before the math of chunk j),
-// and shared by all wavefronts.  The copy is global_load_lds_dwordx4 (no staging registers); tiles are
-// unpadded and XOR-swizzled (gca_mfma.h).
+// (64 x D bf16 each) are read once per workgroup with asynchronous global_load_lds_dwordx4 copies
+// (no staging registers) into ONE K tile and ONE V tile in LDS (unpadded, XOR-swizzled), shared by all
+// wavefronts.  The K tile is refilled for chunk j+1 as soon as the S phase of chunk j is over, the V
+// tile after its P.V phase; in-order load retirement lets a wavefront wait for the older copy only,
+// so both refills hide behind the other phase and LDS stays at 32*D bytes per workgroup (4 waves/SIMD
+// at D = 64).
 //
 // Per wavefront and chunk (v_mfma_f32_32x32x16_bf16, lane = (n = lane % 32, h = lane / 32)):
 //   S^T = K_j Q^T   A = K rows from LDS (16-byte reads), B = Q held in registers for the whole

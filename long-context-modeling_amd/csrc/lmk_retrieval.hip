@@ -34,15 +34,6 @@ template <> __device__ __forceinline__ float finish_score<bf16_t>(float dot, flo
     return bf16_bits_to_f(f_to_bf16_bits(r1 / sqrt_hidden));
 }
 
-__device__ __forceinline__ void unpack16(const uint4& raw, float (&out)[8]) {
-    const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        out[2 * i] = __uint_as_float(u[i] << 16);
-        out[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
-    }
-}
-
 // One wavefront per candidate landmark e; all C (<= SCAN_MAX_C) query rows of the sequence
 // sit in LDS as floats.  Requires Dm % (16 / sizeof(T)) == 0.
 constexpr int SCAN_MAX_C = 4;
