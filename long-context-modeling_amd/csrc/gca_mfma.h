@@ -63,20 +63,20 @@ struct TrLane {
     }
 };
 
-// Asynchronous global -> LDS copy of a 64 x D bf16 tile (rows `rs` elements apart in global memory)
+// Asynchronous global -> LDS copy of a ROWS x D bf16 tile (rows `rs` elements apart in global memory)
 // into a swizzled LDS tile, with global_load_lds_dwordx4: lane l of an instruction deposits its 16 bytes
 // at lds_base + 16*l, so one instruction fills 1 KB = 64*16/RB consecutive tile rows.  The swizzle is
 // applied on the source side: the lane that writes physical piece pp of row r fetches logical piece
 // pp ^ swz(r).  Within a row the lanes still cover one contiguous 2*D-byte span of global memory.
 // No staging registers, no ds_write; completion is tracked by vmcnt (wait_async_tiles()).
-template <int D, int NT>
+template <int D, int NT, int ROWS = 64>
 struct TileLoader {
     static constexpr int RB = D * 2;
     static constexpr int PPR = RB / 16;             // 16-byte pieces per row
     static constexpr int RPI = 64 / PPR;            // rows per instruction
     static constexpr int NW = NT / 64;              // wavefronts sharing the copy
-    static constexpr int NI = 64 / RPI / NW;        // instructions per wavefront per tile
-    static_assert(NI >= 1 && NI * RPI * NW == 64, "tile must split evenly over the wavefronts");
+    static constexpr int NI = ROWS / RPI / NW;      // instructions per wavefront per tile
+    static_assert(NI >= 1 && NI * RPI * NW == ROWS, "tile must split evenly over the wavefronts");
     int goff[NI];      // element offset of this lane's piece in instruction i
     int wave;
     __device__ __forceinline__ TileLoader(int tid, int rs) {
@@ -108,11 +108,12 @@ __device__ __forceinline__ void async_row64(const float* src, float* lds_dst, in
 // all outstanding global_load_lds of this wavefront have landed (vmcnt = 0; other counters untouched)
 __device__ __forceinline__ void wait_async_tiles() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 // all but the NEWEST most recent vector-memory operations of this wavefront have completed (loads
-// retire in order, so everything issued before the last NEWEST instructions has landed); NEWEST <= 15
+// retire in order, so everything issued before the last NEWEST instructions has landed).  vmcnt is a
+// 6-bit field split over bits 3:0 and 15:14 of the immediate.
 template <int NEWEST>
 __device__ __forceinline__ void wait_async_tiles_but() {
-    static_assert(NEWEST >= 0 && NEWEST <= 15, "vmcnt immediate");
-    __builtin_amdgcn_s_waitcnt(0x0F70 | NEWEST);
+    static_assert(NEWEST >= 0 && NEWEST <= 63, "vmcnt immediate");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (NEWEST & 15) | ((NEWEST >> 4) << 14));
 }
 
 // XCD-aware work order.  The hardware deals workgroups round-robin to the 8 XCDs (workgroup i runs
