@@ -48,7 +48,7 @@ enum gca_status {
 };
 
 /* Which kernel family a call may use.  AUTO picks the MFMA kernels when the shape
- * qualifies (bf16, K_CTX == 64, D in {64, 128}, Q_CTX % 64 == 0) and the generic
+ * qualifies (bf16, K_CTX == 64, D in {64, 128}; the backward also needs Q_CTX % 64 == 0) and the generic
  * ones otherwise; the other two force a family (MFMA returns GCA_ERR_UNSUPPORTED
  * when the shape does not qualify). */
 enum gca_path { GCA_PATH_AUTO = 0, GCA_PATH_GENERIC = 1, GCA_PATH_MFMA = 2 };
@@ -91,8 +91,30 @@ typedef struct lmk_desc {
     int32_t Dm;             /* landmark width */
     int32_t causal;         /* 1: row c sees chunk e iff (E - C + c) > e, others are -inf */
     float hidden_size;      /* scores are divided by sqrt(hidden_size) */
-    int32_t reserved;
+    int32_t lmk_k_rows;     /* landmark rows allocated per sequence in lmk_k: sequence n starts at row
+                               n * lmk_k_rows (a cache with spare capacity); 0 means E (dense).  Honoured by
+                               lmk_score and lmk_score_topk; lmk_weights_bwd needs the dense form */
 } lmk_desc;
+
+/* What chunk_cache_append does with the last row of every chunk it stores (the landmark position). */
+enum chunk_lmk_row {
+    CHUNK_LMK_KEEP = 0,   /* source chunks have S rows, stored as they are */
+    CHUNK_LMK_ZERO = 1,   /* source chunks have S rows, the last one is stored as zeros */
+    CHUNK_LMK_DROP = 2    /* source chunks have S + 1 rows, the last one is not stored */
+};
+
+typedef struct chunk_cache_desc {
+    int32_t dtype;          /* gca_dtype of the chunks and the landmarks */
+    int32_t lmk_row;        /* chunk_lmk_row */
+    int64_t N;              /* sequences */
+    int64_t capacity;       /* chunks allocated per sequence in k_cache, v_cache and lmk_cache */
+    int64_t count;          /* chunks each sequence already holds = first slot written */
+    int64_t n_new;          /* chunks appended per sequence */
+    int32_t S;              /* rows per stored chunk */
+    int32_t Dm;             /* width of a K/V row, Hkv*D */
+    int32_t Dl;             /* width of a landmark */
+    int32_t reserved;
+} chunk_cache_desc;
 
 /* Library version (major*10000 + minor*100 + patch) and status text. */
 int gca_version(void);
@@ -164,6 +186,15 @@ size_t lmk_weights_bwd_workspace_bytes(const lmk_desc* desc);
 int lmk_weights_bwd(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, const int64_t* indices,
                     const float* weights, const float* dweights, void* dlmk_q, void* dlmk_k,
                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* Stores n_new chunks per sequence into slots count .. count+n_new-1 of a chunk cache that has room for
+ * `capacity` chunks per sequence, so a growing context costs one copy of the new chunks only.
+ * src_k, src_v (N, n_new, S or S+1, Dm); src_lmk (N, n_new, Dl); k_cache, v_cache (N, capacity, S, Dm);
+ * lmk_cache (N, capacity, Dl).  src_lmk / lmk_cache may both be NULL (landmarks kept elsewhere).
+ * Replaces ChunkKVManager.append (model/DRT.py:87-132: a torch.cat of the whole cache per call) together
+ * with the landmark-row handling before it (model/DRT.py:769-779, decode copy :804-813). */
+int chunk_cache_append(const chunk_cache_desc* desc, const void* src_k, const void* src_v, const void* src_lmk,
+                       void* k_cache, void* v_cache, void* lmk_cache, void* stream);
 
 #ifdef __cplusplus
 }

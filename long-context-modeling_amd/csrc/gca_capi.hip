@@ -25,14 +25,16 @@ int check_lmk(const lmk_desc* d) {
     if (d == nullptr) return GCA_ERR_NULL;
     if (d->dtype != GCA_F32 && d->dtype != GCA_BF16) return GCA_ERR_DTYPE;
     if (d->N <= 0 || d->C <= 0 || d->E <= 0 || d->Dm <= 0 || d->topk <= 0) return GCA_ERR_SHAPE;
+    if (d->E > INT32_MAX) return GCA_ERR_SHAPE;
+    if (d->lmk_k_rows != 0 && d->lmk_k_rows < d->E) return GCA_ERR_SHAPE;
     if (d->causal && d->C > d->E) return GCA_ERR_SHAPE;
     if (!(d->hidden_size > 0.f)) return GCA_ERR_SHAPE;
     return GCA_OK;
 }
 
 // returns GCA_OK and sets use_mfma, or an error
-int pick_path(const gca_desc& d, bool& use_mfma) {
-    const bool ok = mfma_supported(d);
+int pick_path(const gca_desc& d, bool& use_mfma, bool forward) {
+    const bool ok = forward ? mfma_fwd_supported(d) : mfma_supported(d);
     if (d.path == GCA_PATH_MFMA && !ok) return GCA_ERR_UNSUPPORTED;
     use_mfma = (d.path != GCA_PATH_GENERIC) && ok;
     return GCA_OK;
@@ -63,7 +65,7 @@ int gca_fwd(const gca_desc* desc, const void* q, const void* k, const void* v, c
     if (rc != GCA_OK) return rc;
     if (!q || !k || !v || !weights || !o) return GCA_ERR_NULL;
     bool use_mfma = false;
-    if ((rc = pick_path(*desc, use_mfma)) != GCA_OK) return rc;
+    if ((rc = pick_path(*desc, use_mfma, true)) != GCA_OK) return rc;
     if (use_mfma) return launch_fwd_mfma(*desc, false, q, k, v, nullptr, weights, o, lse, (hipStream_t)stream);
     return launch_fwd_generic(*desc, false, q, k, v, nullptr, weights, o, lse, (hipStream_t)stream);
 }
@@ -82,7 +84,7 @@ int gca_bwd(const gca_desc* desc, const void* q, const void* k, const void* v, c
     if (!q || !k || !v || !weights || !dout || !lse || !dq || !dk || !dv || !dw) return GCA_ERR_NULL;
     if (!workspace || workspace_bytes < gca_bwd_workspace_bytes(desc)) return GCA_ERR_WORKSPACE;
     bool use_mfma = false;
-    if ((rc = pick_path(*desc, use_mfma)) != GCA_OK) return rc;
+    if ((rc = pick_path(*desc, use_mfma, false)) != GCA_OK) return rc;
     if (use_mfma)
         return launch_bwd_mfma(*desc, false, q, k, v, nullptr, weights, dout, lse, dq, dk, dv, dw, (float*)workspace,
                                (hipStream_t)stream);
@@ -96,7 +98,7 @@ int gca_fwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, co
     if (rc != GCA_OK) return rc;
     if (!q || !k_cache || !v_cache || !indices || !weights || !o) return GCA_ERR_NULL;
     bool use_mfma = false;
-    if ((rc = pick_path(*desc, use_mfma)) != GCA_OK) return rc;
+    if ((rc = pick_path(*desc, use_mfma, true)) != GCA_OK) return rc;
     if (use_mfma) return launch_fwd_mfma(*desc, true, q, k_cache, v_cache, indices, weights, o, lse, (hipStream_t)stream);
     return launch_fwd_generic(*desc, true, q, k_cache, v_cache, indices, weights, o, lse, (hipStream_t)stream);
 }
@@ -111,7 +113,7 @@ int gca_bwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, co
         return GCA_ERR_NULL;
     if (!workspace || workspace_bytes < gca_bwd_workspace_bytes(desc)) return GCA_ERR_WORKSPACE;
     bool use_mfma = false;
-    if ((rc = pick_path(*desc, use_mfma)) != GCA_OK) return rc;
+    if ((rc = pick_path(*desc, use_mfma, false)) != GCA_OK) return rc;
     if (use_mfma)
         return launch_bwd_mfma(*desc, true, q, k_cache, v_cache, indices, weights, dout, lse, dq, dk_cache, dv_cache, dw,
                                (float*)workspace, (hipStream_t)stream);
@@ -158,8 +160,22 @@ int lmk_weights_bwd(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, 
     int rc = check_lmk(desc);
     if (rc != GCA_OK) return rc;
     if (!lmk_q || !lmk_k || !indices || !weights || !dweights || !dlmk_q || !dlmk_k) return GCA_ERR_NULL;
+    if (desc->lmk_k_rows != 0 && desc->lmk_k_rows != desc->E) return GCA_ERR_UNSUPPORTED;
     return launch_lmk_bwd(*desc, lmk_q, lmk_k, indices, weights, dweights, dlmk_q, dlmk_k, workspace, workspace_bytes,
                           (hipStream_t)stream);
+}
+
+int chunk_cache_append(const chunk_cache_desc* d, const void* src_k, const void* src_v, const void* src_lmk,
+                       void* k_cache, void* v_cache, void* lmk_cache, void* stream) {
+    if (d == nullptr) return GCA_ERR_NULL;
+    if (d->dtype != GCA_F32 && d->dtype != GCA_BF16) return GCA_ERR_DTYPE;
+    if (d->lmk_row != CHUNK_LMK_KEEP && d->lmk_row != CHUNK_LMK_ZERO && d->lmk_row != CHUNK_LMK_DROP) return GCA_ERR_SHAPE;
+    if (d->N <= 0 || d->capacity <= 0 || d->count < 0 || d->n_new <= 0 || d->S <= 0 || d->Dm <= 0) return GCA_ERR_SHAPE;
+    if (d->count + d->n_new > d->capacity) return GCA_ERR_SHAPE;
+    if (!src_k || !src_v || !k_cache || !v_cache) return GCA_ERR_NULL;
+    if ((src_lmk == nullptr) != (lmk_cache == nullptr)) return GCA_ERR_NULL;
+    if (src_lmk != nullptr && d->Dl <= 0) return GCA_ERR_SHAPE;
+    return launch_chunk_append(*d, src_k, src_v, src_lmk, k_cache, v_cache, lmk_cache, (hipStream_t)stream);
 }
 
 }  // extern "C"

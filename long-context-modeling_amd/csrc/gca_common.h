@@ -84,7 +84,8 @@ int launch_fwd_generic(const gca_desc& d, bool indexed, const void* q, const voi
 int launch_bwd_generic(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v,
                        const int64_t* indices, const void* w, const void* dout, const float* lse,
                        void* dq, void* dk, void* dv, float* dw, float* delta, hipStream_t s);
-bool mfma_supported(const gca_desc& d);
+bool mfma_supported(const gca_desc& d);       // forward and backward
+bool mfma_fwd_supported(const gca_desc& d);   // forward only: any Q_CTX
 int launch_fwd_mfma(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v,
                     const int64_t* indices, const void* w, void* o, float* lse, hipStream_t s);
 int launch_bwd_mfma(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v,
@@ -98,6 +99,8 @@ size_t lmk_bwd_ws_bytes(const lmk_desc& d);
 int launch_lmk_bwd(const lmk_desc& d, const void* lq, const void* lk, const int64_t* idx, const float* w,
                    const float* dw, void* dlq, void* dlk, void* wsp, size_t ws_bytes, hipStream_t s);
 size_t bwd_workspace_bytes(const gca_desc& d, bool indexed);
+int launch_chunk_append(const chunk_cache_desc& d, const void* sk, const void* sv, const void* sl,
+                        void* dk, void* dv, void* dl, hipStream_t s);
 int launch_dw(const Params& p, const float* delta, float* dw, hipStream_t s);
 // bytes of the per-chunk row sums D_j at the start of the backward workspace (256-byte multiple)
 inline size_t delta_bytes(const Params& p) {

@@ -1,6 +1,8 @@
 // GCA forward on the gfx950 matrix cores (bf16 in, fp32 accumulate).
 //
-// Shape class: bf16, K_CTX == 64, D in {64, 128}, Q_CTX % 64 == 0, sm_scale > 0.
+// Shape class: bf16, K_CTX == 64, D in {64, 128}, sm_scale > 0; any Q_CTX (the rows a 64-row query tile
+// has beyond Q_CTX are computed on zeros and never stored, so a decode step of 1 or 2 rows streams its
+// retrieved chunks exactly like a full chunk does).
 //
 // Work split.  A workgroup owns one (z, kv head, slice of GS query heads of the group, 64-row
 // query tile) and walks the K retrieved chunks.  It has 2*GS wavefronts; wavefront w owns the
@@ -43,7 +45,7 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
     const int n = lane & 31, h = lane >> 5;
     const int gs = wave >> 1, qb = wave & 1;
 
-    const int nqt = p.Q_CTX / 64;
+    const int nqt = (p.Q_CTX + 63) / 64;
     const int nslice = p.G / GS;
     // logical order: (sequence n, kv head, head slice) pair-major, then the pair's rows (z in n, q tile)
     const int64_t rows = p.zpn * nqt;
@@ -60,10 +62,12 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
 
     // Q as the B operand: lane holds row n, dims 16*ks + 8*h .. +7
     bf16x8 qB[KS];
+    const bool row_ok = q0 + n < p.Q_CTX;      // false only in the last tile of a Q_CTX that is not a multiple of 64
     {
         const uint16_t* qp = q + ((z * p.Hq + hq) * (int64_t)p.Q_CTX + q0 + n) * D + 8 * h;
+        const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qB[ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
+        for (int ks = 0; ks < KS; ++ks) qB[ks] = row_ok ? *reinterpret_cast<const bf16x8*>(qp + 16 * ks) : zero8;
     }
 
     f32x16 oacc[DB];
@@ -138,7 +142,7 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
         const float l = sum + p.sm_n * __builtin_amdgcn_exp2f(-m2);
         const float wj = w_is_bf16 ? bf16_bits_to_f(((const uint16_t*)w)[z * p.K + j]) : ((const float*)w)[z * p.K + j];
         const float inv = wj / l;
-        if (lse != nullptr && h == 0)
+        if (lse != nullptr && h == 0 && row_ok)
             lse[((z * p.Hq + hq) * (int64_t)p.K + j) * p.Q_CTX + q0 + n] = m2 + __builtin_amdgcn_logf(l);
 
         // ---- P~ as the A operand: step t4 covers keys 16*t4 .. +15; slots 0-3 = keys 16*t4 + 4h + c,
@@ -179,18 +183,21 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
         for (int r = 0; r < 16; ++r) {
             const int row = 8 * (r >> 2) + 4 * h + (r & 3);
             const __bf16 ob = (__bf16)oacc[db][r];
-            op[row * D + 32 * db + n] = __builtin_bit_cast(uint16_t, ob);
+            if (q0 + row < p.Q_CTX) op[row * D + 32 * db + n] = __builtin_bit_cast(uint16_t, ob);
         }
 }
 
-bool mfma_supported(const gca_desc& d) {
-    return d.dtype == GCA_BF16 && d.K_CTX == 64 && (d.D == 64 || d.D == 128) && d.Q_CTX % 64 == 0 && d.sm_scale > 0.f;
+bool mfma_fwd_supported(const gca_desc& d) {
+    return d.dtype == GCA_BF16 && d.K_CTX == 64 && (d.D == 64 || d.D == 128) && d.sm_scale > 0.f;
 }
+
+// the backward kernels walk whole 64-row query tiles
+bool mfma_supported(const gca_desc& d) { return mfma_fwd_supported(d) && d.Q_CTX % 64 == 0; }
 
 template <int D, int GS>
 static int launch_gs(const Params& p, const void* q, const void* k, const void* v, const int64_t* idx,
                      const void* w, int w_is_bf16, void* o, float* lse, hipStream_t s) {
-    const int64_t blocks = xcd_grid(p.Z * p.Hkv * (p.G / GS) * (p.Q_CTX / 64));
+    const int64_t blocks = xcd_grid(p.Z * p.Hkv * (p.G / GS) * ((p.Q_CTX + 63) / 64));
     if (blocks <= 0 || blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
     if (p.indexed)
         hipLaunchKernelGGL((gca_fwd_mfma_kernel<D, GS, true>), dim3((unsigned)blocks), dim3(128 * GS), 0, s, p,
@@ -211,7 +218,7 @@ static int launch_d(const Params& p, const void* q, const void* k, const void* v
 
 int launch_fwd_mfma(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v,
                     const int64_t* indices, const void* w, void* o, float* lse, hipStream_t s) {
-    if (!mfma_supported(d)) return GCA_ERR_UNSUPPORTED;
+    if (!mfma_fwd_supported(d)) return GCA_ERR_UNSUPPORTED;
     const Params p = make_params(d, indexed);
     const int wb = d.w_dtype == GCA_BF16 ? 1 : 0;
     if (d.D == 64) return launch_d<64>(p, q, k, v, indices, w, wb, o, lse, s);

@@ -66,7 +66,7 @@ lmk_score_scan_kernel(lmk_desc d, const T* __restrict__ lq, const T* __restrict_
 #pragma unroll
             for (int a = 0; a < SCAN_EPW; ++a) {
                 const int64_t e = min(e0 + a, d.E - 1);          // the tail re-reads the last landmark
-                raw[a] = *reinterpret_cast<const u32x4*>(lk + (n * d.E + e) * Dm + (int64_t)iv * VN);
+                raw[a] = *reinterpret_cast<const u32x4*>(lk + (n * d.lmk_k_rows + e) * Dm + (int64_t)iv * VN);
             }
 #pragma unroll
             for (int a = 0; a < SCAN_EPW; ++a) {
@@ -139,7 +139,7 @@ lmk_score_scan_mfma_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const ui
         const int64_t e0 = (((int64_t)blockIdx.x * steps + step) * 4 + wave) * 32;
         if (e0 >= d.E) break;
         const int64_t erow = min(e0 + n32, d.E - 1);                    // the tail re-reads the last landmark
-        const uint16_t* bptr = lk + (nb * d.E + erow) * Dm + 8 * h;
+        const uint16_t* bptr = lk + (nb * d.lmk_k_rows + erow) * Dm + 8 * h;
         f32x16 acc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[r] = 0.f;
@@ -207,8 +207,8 @@ lmk_score_mfma_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const uint16_
         const int row = (i * 4 + wave) * 8 + lane / 8;
         const int lp = (lane % 8) ^ swz(row);
         aoff[i] = (nb * d.C + min(c0 + row, d.C - 1)) * d.Dm + lp * 8;          // tail rows re-read the last row
-        b0off[i] = (nb * d.E + min(e0 + row, d.E - 1)) * d.Dm + lp * 8;
-        b1off[i] = (nb * d.E + min(e0 + 64 + row, d.E - 1)) * d.Dm + lp * 8;
+        b0off[i] = (nb * d.lmk_k_rows + min(e0 + row, d.E - 1)) * d.Dm + lp * 8;
+        b1off[i] = (nb * d.lmk_k_rows + min(e0 + 64 + row, d.E - 1)) * d.Dm + lp * 8;
     }
     typedef __attribute__((address_space(3))) void lds_void;
     typedef __attribute__((address_space(1))) const void gbl_void;
@@ -283,7 +283,7 @@ lmk_score_tile_kernel(lmk_desc d, const T* __restrict__ lq, const T* __restrict_
                 const int rr = i >> 5, kk = i & 31;
                 const bool kin = (k0 + kk) < d.Dm;
                 sA[rr][kk] = (kin && (c0 + rr) < d.C) ? to_f(lq[(n * d.C + c0 + rr) * d.Dm + k0 + kk]) : 0.f;
-                sB[rr][kk] = (kin && (e0 + rr) < d.E) ? to_f(lk[(n * d.E + e0 + rr) * d.Dm + k0 + kk]) : 0.f;
+                sB[rr][kk] = (kin && (e0 + rr) < d.E) ? to_f(lk[(n * d.lmk_k_rows + e0 + rr) * d.Dm + k0 + kk]) : 0.f;
             }
             __syncthreads();
 #pragma unroll
@@ -346,7 +346,9 @@ static int launch_score_t(const lmk_desc& d, const void* lq, const void* lk, voi
     return hipGetLastError() == hipSuccess ? GCA_OK : GCA_ERR_LAUNCH;
 }
 
-int launch_lmk_score(const lmk_desc& d, const void* lq, const void* lk, void* scores, hipStream_t s) {
+int launch_lmk_score(const lmk_desc& d_in, const void* lq, const void* lk, void* scores, hipStream_t s) {
+    lmk_desc d = d_in;
+    if (d.lmk_k_rows == 0) d.lmk_k_rows = (int32_t)d.E;   // the kernels always stride by lmk_k_rows
     if (d.dtype == GCA_F32) return launch_score_t<float>(d, lq, lk, scores, s);
     if (d.dtype == GCA_BF16) return launch_score_t<bf16_t>(d, lq, lk, scores, s);
     return GCA_ERR_DTYPE;

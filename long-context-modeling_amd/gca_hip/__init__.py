@@ -2,8 +2,10 @@
 from . import _lib
 from .gca import attention, gca_kv_cache, attention_indexed, gca_kv_cache_indexed
 from .retrieval import landmark_scores, landmark_topk, landmark_retrieve, gather_chunks, gca_layer
+from .chunk_cache import ChunkKVManager, chunk_cache_append
 
 __all__ = [
     "attention", "gca_kv_cache", "attention_indexed", "gca_kv_cache_indexed",
     "landmark_scores", "landmark_topk", "landmark_retrieve", "gather_chunks", "gca_layer",
+    "ChunkKVManager", "chunk_cache_append",
 ]

@@ -20,8 +20,9 @@ GCA_OK = 0
 SYMBOLS = (
     "gca_version", "gca_strerror", "gca_fwd", "gca_bwd_workspace_bytes", "gca_bwd", "gca_fwd_indexed",
     "gca_bwd_indexed", "lmk_score", "lmk_topk_workspace_bytes", "lmk_topk", "lmk_score_topk",
-    "lmk_weights_bwd_workspace_bytes", "lmk_weights_bwd",
+    "lmk_weights_bwd_workspace_bytes", "lmk_weights_bwd", "chunk_cache_append",
 )
+CHUNK_LMK_KEEP, CHUNK_LMK_ZERO, CHUNK_LMK_DROP = 0, 1, 2
 
 
 class GcaDesc(ctypes.Structure):
@@ -40,7 +41,15 @@ class LmkDesc(ctypes.Structure):
         ("dtype", ctypes.c_int32), ("topk", ctypes.c_int32),
         ("N", ctypes.c_int64), ("C", ctypes.c_int64), ("E", ctypes.c_int64),
         ("Dm", ctypes.c_int32), ("causal", ctypes.c_int32),
-        ("hidden_size", ctypes.c_float), ("reserved", ctypes.c_int32),
+        ("hidden_size", ctypes.c_float), ("lmk_k_rows", ctypes.c_int32),
+    ]
+
+
+class ChunkCacheDesc(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int32), ("lmk_row", ctypes.c_int32),
+        ("N", ctypes.c_int64), ("capacity", ctypes.c_int64), ("count", ctypes.c_int64), ("n_new", ctypes.c_int64),
+        ("S", ctypes.c_int32), ("Dm", ctypes.c_int32), ("Dl", ctypes.c_int32), ("reserved", ctypes.c_int32),
     ]
 
 
@@ -77,6 +86,8 @@ def _declare(lib):
     lib.lmk_weights_bwd_workspace_bytes.argtypes = [L]
     lib.lmk_weights_bwd.restype = ctypes.c_int
     lib.lmk_weights_bwd.argtypes = [L, P, P, I64P, FP, FP, P, P, P, ctypes.c_size_t, P]
+    lib.chunk_cache_append.restype = ctypes.c_int
+    lib.chunk_cache_append.argtypes = [ctypes.POINTER(ChunkCacheDesc), P, P, P, P, P, P, P]
 
 
 def lib():

@@ -14,22 +14,35 @@ from . import _lib
 from .gca import _DT, _ptr, _stream
 
 
-def _lmk_desc(dtype, topk, N, C, E, Dm, causal, hidden_size):
+def _lmk_desc(dtype, topk, N, C, E, Dm, causal, hidden_size, lmk_k_rows=0):
     return _lib.LmkDesc(dtype=_DT[dtype], topk=int(topk), N=N, C=C, E=E, Dm=Dm, causal=1 if causal else 0,
-                        hidden_size=float(hidden_size), reserved=0)
+                        hidden_size=float(hidden_size), lmk_k_rows=int(lmk_k_rows))
+
+
+def _dense_or_strided(lmk_k):
+    """(tensor, rows per sequence) for the scoring kernel: the first E landmarks of a store allocated
+    with spare capacity (``store[:, :E]``) are read in place, anything else is made contiguous."""
+    N, E, Dm = lmk_k.shape
+    if lmk_k.is_contiguous():
+        return lmk_k, 0
+    s0, s1, s2 = lmk_k.stride()
+    if s2 == 1 and s1 == Dm and s0 % Dm == 0 and s0 // Dm >= E and s0 // Dm < 2 ** 31:
+        return lmk_k, s0 // Dm
+    return lmk_k.contiguous(), 0
 
 
 def landmark_scores(lmk_q, lmk_k, hidden_size=None, causal=True):
     """scores[n,c,e] = <lmk_q[n,c], lmk_k[n,e]> / sqrt(hidden), -inf where not strictly past
     (model/DRT.py:612-613)."""
     assert lmk_q.is_cuda and lmk_q.dim() == 3 and lmk_k.dim() == 3 and lmk_q.dtype in _DT and lmk_k.dtype == lmk_q.dtype
-    lmk_q, lmk_k = lmk_q.contiguous(), lmk_k.contiguous()
+    lmk_q = lmk_q.contiguous()
+    lmk_k, rows = _dense_or_strided(lmk_k)
     N, C, Dm = lmk_q.shape
     E = lmk_k.shape[1]
     assert lmk_k.shape[0] == N and lmk_k.shape[2] == Dm
     hidden_size = Dm if hidden_size is None else hidden_size
     scores = torch.empty((N, C, E), device=lmk_q.device, dtype=lmk_q.dtype)
-    desc = _lmk_desc(lmk_q.dtype, 1, N, C, E, Dm, causal, hidden_size)
+    desc = _lmk_desc(lmk_q.dtype, 1, N, C, E, Dm, causal, hidden_size, rows)
     with torch.cuda.device(lmk_q.device):
         rc = _lib.lib().lmk_score(ctypes.byref(desc), _ptr(lmk_q), _ptr(lmk_k), _ptr(scores), _stream(lmk_q.device))
     _lib.check(rc, "lmk_score")
@@ -97,6 +110,11 @@ def landmark_retrieve(lmk_q, lmk_k, topk, hidden_size=None, causal=True, noise=N
     gradient to ``lmk_q`` and ``lmk_k``."""
     assert lmk_q.is_cuda and lmk_q.dim() == 3 and lmk_k.dim() == 3
     hidden_size = lmk_q.shape[-1] if hidden_size is None else hidden_size
+    if not (torch.is_grad_enabled() and (lmk_q.requires_grad or lmk_k.requires_grad)):
+        # inference: no copy of a landmark store that is a view with spare capacity
+        scores = landmark_scores(lmk_q, lmk_k, hidden_size, causal)
+        indices, weights = landmark_topk(scores, topk, causal, noise)
+        return scores, indices, weights
     return _Retrieve.apply(lmk_q, lmk_k, topk, hidden_size, causal, noise)
 
 

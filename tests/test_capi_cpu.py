@@ -79,3 +79,63 @@ def test_missing_library_is_an_error(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libgca_hip.so")
     with pytest.raises(RuntimeError):
         _lib.lib()
+
+
+def test_chunk_cache_desc_layout_and_validation():
+    """struct chunk_cache_desc is 56 bytes with the header's field order; bad requests are refused before
+    any launch (no GPU needed)."""
+    import ctypes
+    from gca_hip import _lib
+    assert ctypes.sizeof(_lib.ChunkCacheDesc) == 56
+    L = _lib.lib()
+    one = ctypes.c_void_p(16)     # any non-NULL address: validation fails before it is used
+    ok = dict(dtype=0, lmk_row=0, N=1, capacity=4, count=0, n_new=2, S=8, Dm=16, Dl=4, reserved=0)
+
+    def call(**kw):
+        d = _lib.ChunkCacheDesc(**{**ok, **kw})
+        return L.chunk_cache_append(ctypes.byref(d), one, one, one, one, one, one, None)
+
+    assert call(dtype=5) == 3
+    assert call(lmk_row=3) == 2
+    assert call(count=3) == 2          # 3 + 2 > capacity 4
+    assert call(n_new=0) == 2
+    assert call(Dl=0) == 2
+    d = _lib.ChunkCacheDesc(**ok)
+    assert L.chunk_cache_append(ctypes.byref(d), None, one, one, one, one, one, None) == 1
+    assert L.chunk_cache_append(ctypes.byref(d), one, one, one, one, one, None, None) == 1   # landmarks: both or neither
+    assert L.chunk_cache_append(None, one, one, one, one, one, one, None) == 1
+
+
+def test_lmk_k_rows_validation():
+    import ctypes
+    from gca_hip import _lib
+    L = _lib.lib()
+    one = ctypes.c_void_p(16)
+    d = _lib.LmkDesc(dtype=0, topk=2, N=2, C=1, E=8, Dm=8, causal=1, hidden_size=8.0, lmk_k_rows=4)
+    assert L.lmk_score(ctypes.byref(d), one, one, one, None) == 2          # fewer rows allocated than used
+
+
+def test_manager_state_logic_on_cpu():
+    """The host-only parts of ChunkKVManager (no kernel involved): decode state and hidden-state cache
+    follow model/DRT.py:141-191."""
+    import torch
+    from gca_hip import ChunkKVManager
+    m = ChunkKVManager(group_size=2)
+    assert m.chunk_k is None and m.past_lmk_embeds is None and m.count == 0 and m.capacity == 0
+    assert m.current_retrieved_chunk(1) == (None, None, None)
+    idx = torch.arange(24).reshape(2, 4, 3)
+    w = torch.rand(2, 4, 3)
+    m.update_current_retrieved_chunk(idx, w, 1)
+    i1, w1 = m.current_retrieved_indices(1)
+    assert torch.equal(i1, idx[:, -1]) and torch.equal(w1, w[:, -1:]) and m.current_retrieved_indices(0) == (None, None)
+    m.update_current_retrieved_chunk(idx[:, 0], w[:, :1], 0)               # 2-D ids as the decode step passes them
+    assert torch.equal(m.current_retrieved_indices(0)[0], idx[:, 0])
+    h = torch.rand(2, 3, 5)
+    m.cache_lower_hidden_states(h)
+    m.cache_lower_hidden_states(h[:, :1])
+    assert m.lower_hidden_states.shape == (2, 4, 5) and torch.equal(m.lower_hidden_states[:, 3], h[:, 0])
+    m.clear_lower_hidden_states()
+    assert m.lower_hidden_states is None
+    import pytest
+    with pytest.raises(AssertionError):
+        m.append(torch.zeros(1, 1, 8, 16), torch.zeros(1, 1, 8, 16), torch.zeros(1, 1, 4))   # CPU tensors: no fallback

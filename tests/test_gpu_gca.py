@@ -101,6 +101,9 @@ def test_reference_decode_recipe(Q):
     (2, 2, 1, 2, 64, 48, 256),
     (5, 6, 3, 1, 1, 64, 64),      # single query row, single retrieved chunk
     (2, 2, 2, 4, 128, 64, 64),    # two 64-row tiles per chunk
+    (2, 4, 2, 3, 100, 64, 64),    # bf16: matrix-core forward with a partial last tile, generic backward
+    (2, 4, 2, 3, 96, 64, 64),     # the last tile's second half is empty
+    (3, 8, 2, 4, 2, 64, 128),     # decode step, 4 query heads per kv head, d=128
 ])
 def test_shapes_generic_and_auto(shape, dtype):
     Z, Hq, Hkv, K, Q, S, d = shape

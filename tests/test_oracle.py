@@ -249,3 +249,59 @@ def test_layer_row_shift_and_zero_first_chunk():
                     p = ex / (1.0 + ex.sum(-1, keepdim=True))
                     ref[h] += w[n, c, j] * (p @ cv[n, e, :, h * d:(h + 1) * d])
             assert torch.allclose(out[n, c + 1], ref, atol=1e-5)
+
+
+# ----------------------------------------------------------------------------- chunk cache + decode flow
+
+def _flow_inputs(N, C, Hq, Hkv, S, d, Dl, seed):
+    q_all = _rand(N, C, Hq, S, d, seed=seed, scale=0.5)
+    ck = _rand(N, C, S, Hkv * d, seed=seed + 1, scale=0.5)
+    cv = _rand(N, C, S, Hkv * d, seed=seed + 2, scale=0.5)
+    lq, lk = _rand(N, C, Dl, seed=seed + 3), _rand(N, C, Dl, seed=seed + 4)
+    return q_all, ck, cv, lq, lk
+
+
+@pytest.mark.parametrize("steps", [(1,), (2,), (1, 2, 5)])
+@pytest.mark.parametrize("prompt", [1, 3])
+def test_generation_reproduces_batch_form(steps, prompt):
+    """Chunk-by-chunk generation == the batch layer on the whole sequence, position for position (the
+    self-consistency tests/generation_unittest.py of the reference asserts).  Breaks on a wrong row shift,
+    a wrong visible set for the single decode row, a stale retrieval state or a wrong cache slot."""
+    from oracle import cache_oracle as co
+    N, C, Hq, Hkv, S, d, Dl, topk = 2, 7, 4, 2, 8, 16, 12, 3
+    q_all, ck, cv, lq, lk = _flow_inputs(N, C, Hq, Hkv, S, d, Dl, seed=40)
+    full, idx_full, _ = orc.gca_layer(q_all, ck, cv, lq, lk, topk, Hkv, sm_n=1.0)
+    out, picked = co.generate(q_all, ck, cv, lq, lk, topk, Hkv, prompt, sm_n=1.0, steps=steps)
+    assert torch.equal(out[:, :prompt], torch.zeros_like(out[:, :prompt]))
+    assert (out[:, prompt:] - full[:, prompt:]).abs().max().item() < 1e-6      # retrieval weights are float32
+    for i, c in enumerate(range(prompt, C)):
+        kk = picked[i].shape[1]                               # min(chunks stored at that time, topk)
+        assert torch.equal(picked[i], idx_full[:, c - 1, :kk])     # chunk c uses retrieval row c-1
+
+
+def test_cache_oracle_vs_loops():
+    """append / retrieve_chunks / landmark_row against python loops."""
+    from oracle import cache_oracle as co
+    N, S, Dm = 2, 4, 6
+    cache = co.ChunkCacheOracle()
+    parts = [_rand(N, n, S, Dm, seed=50 + n) for n in (2, 1, 3)]
+    for p in parts:
+        cache.append(p, p + 1, p[:, :, 0])
+    C = 6
+    assert cache.chunk_k.shape == (N, C, S, Dm) and cache.lmk_embs.shape == (N, C, Dm)
+    flat = [p[n, i] for n in range(N) for p in parts for i in range(p.shape[1])]
+    for n in range(N):
+        for c in range(C):
+            assert torch.equal(cache.chunk_k[n, c], flat[n * C + c])
+            assert torch.equal(cache.chunk_v[n, c], flat[n * C + c] + 1)
+    idx = torch.tensor([[5, 0, 2], [1, 1, 4]])
+    k, v = cache.retrieve_chunks(idx)
+    for n in range(N):
+        for j in range(3):
+            assert torch.equal(k[n, j], cache.chunk_k[n, idx[n, j]])
+            assert torch.equal(v[n, j], cache.chunk_v[n, idx[n, j]])
+    x = _rand(N, 3, S + 1, Dm, seed=60)
+    z = co.landmark_row(x[:, :, :S], "zero")
+    assert torch.equal(z[:, :, :-1], x[:, :, :S - 1]) and z[:, :, -1].abs().max() == 0
+    assert torch.equal(co.landmark_row(x, "drop"), x[:, :, :S])
+    assert co.landmark_row(x, "keep") is x
