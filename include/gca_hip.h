@@ -14,7 +14,7 @@
  * reference interface it replaces (paths relative to that checkout).
  *
  * Tensor layouts (element type T = desc.dtype; all contiguous):
- *   q, o, do, dq      (Z, Hq, Q_CTX, D)
+ *   q, o, do, dq      (Z, Hq, Q_CTX, D)              or token-major, see gca_q_layout
  *   k, v, dk, dv      (Z, Hkv, K, K_CTX, D)          gathered ("retrieved chunks") form
  *   weights           (Z, K)      type desc.w_dtype  shared by all heads
  *   lse               (Z, Hq, K, Q_CTX)  float       log2 of the softmax denominator of the
@@ -53,6 +53,16 @@ enum gca_status {
  * when the shape does not qualify). */
 enum gca_path { GCA_PATH_AUTO = 0, GCA_PATH_GENERIC = 1, GCA_PATH_MFMA = 2 };
 
+/* Where the rows of q, o, do and dq live (indexed entry points only; the gathered ones take HEAD_MAJOR).
+ * HEAD_MAJOR  (Z, Hq, Q_CTX, D): what the reference's kernels take after its rearrange + contiguous
+ *             (model/DRT.py:372-378).
+ * TOKEN_MAJOR (N, Z/N + q_skip, Q_CTX, Hq*D): the projection's own output, rows of all heads side by
+ *             side; the first q_skip chunks of every sequence are not part of the problem (q_skip = 1
+ *             hands over the whole (N, C, S, Hq*D) tensor although chunk 0 retrieves nothing) and are
+ *             neither read nor written.  Saves the permute copies on both sides of the kernel
+ *             (model/DRT.py:366-378, :384). */
+enum gca_q_layout { GCA_Q_HEAD_MAJOR = 0, GCA_Q_TOKEN_MAJOR = 1 };
+
 /* gca_bwd / gca_bwd_indexed are several launches.  desc.stages selects which of them run
  * (0 = all); a profiler or benchmark can time one stage with events around the call.  Running a
  * later stage alone needs the buffers an earlier stage fills (delta in the workspace). */
@@ -80,6 +90,8 @@ typedef struct gca_desc {
     int32_t stages;     /* bitmask of gca_stage for the backward entry points; 0 = all */
     int64_t N;          /* indexed entry points: sequences in the cache (Z % N == 0) */
     int64_t C;          /* indexed entry points: chunks per sequence in the cache */
+    int32_t q_layout;   /* gca_q_layout of q, o, do, dq */
+    int32_t q_skip;     /* TOKEN_MAJOR: leading chunks of every sequence that are skipped */
 } gca_desc;
 
 typedef struct lmk_desc {

@@ -47,7 +47,7 @@ gca_bwd_dq_generic_kernel(Params p, const T* __restrict__ q, const T* __restrict
     float qreg[DPT], doreg[DPT], dqacc[DPT];
 #pragma unroll
     for (int i = 0; i < DPT; ++i) { qreg[i] = 0.f; doreg[i] = 0.f; dqacc[i] = 0.f; }
-    const int64_t qoff = ((z * p.Hq + h) * (int64_t)p.Q_CTX + row) * D + t * DPT;
+    const int64_t qoff = q_base(p, z, h) + row * p.q_rs + t * DPT;
     if (row_ok) {
 #pragma unroll
         for (int i = 0; i < DPT; ++i) { qreg[i] = to_f(q[qoff + i]); doreg[i] = to_f(dout[qoff + i]); }
@@ -173,7 +173,7 @@ gca_bwd_dkdv_generic_kernel(Params p, const T* __restrict__ q, const T* __restri
     const float wj = to_f(w[z * p.K + j]);
     for (int g = 0; g < p.G; ++g) {
         const int h = hk * p.G + g;
-        const int64_t qbase = (z * p.Hq + h) * (int64_t)p.Q_CTX;
+        const int64_t qbase = q_base(p, z, h);
         const int64_t lbase = ((z * p.Hq + h) * (int64_t)p.K + j) * p.Q_CTX;
         for (int q0 = 0; q0 < p.Q_CTX; q0 += QT) {
             __syncthreads();
@@ -182,8 +182,8 @@ gca_bwd_dkdv_generic_kernel(Params p, const T* __restrict__ q, const T* __restri
                 const int gq = q0 + qq;
                 float a = 0.f, b = 0.f;
                 if (gq < p.Q_CTX) {
-                    a = to_f(q[(qbase + gq) * D + dd]);
-                    b = to_f(dout[(qbase + gq) * D + dd]);
+                    a = to_f(q[qbase + gq * p.q_rs + dd]);
+                    b = to_f(dout[qbase + gq * p.q_rs + dd]);
                 }
                 sQ[i] = a;
                 sDO[i] = b;

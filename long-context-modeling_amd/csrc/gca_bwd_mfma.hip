@@ -70,9 +70,10 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
     const int hq = hk * p.G + slice * GS + gs;
     const int q0 = qt * 64 + qb * 32;
 
+    const int qrs = (int)p.q_rs;               // row stride of q / dO / dq in elements
     bf16x8 qB[KS], doB[KS];
     {
-        const int64_t off = ((z * p.Hq + hq) * (int64_t)p.Q_CTX + q0 + n) * D + 8 * h;
+        const int64_t off = q_base_n(p, nseq, z, hq) + (q0 + n) * qrs + 8 * h;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             qB[ks] = *reinterpret_cast<const bf16x8*>(q + off + 16 * ks);
@@ -171,13 +172,16 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
         __syncthreads();
     }
 
-    uint16_t* dqp = dq + ((z * p.Hq + hq) * (int64_t)p.Q_CTX + q0) * D;
+    // register r of block db is row 8*(r/4) + 4*h + r%4, column 32*db + n: a wavefront-uniform base per
+    // (r, db) plus one 32-bit lane offset, so the 32 stores share their address arithmetic
+    uint16_t* dqp = dq + q_base_n(p, nseq, z, hq) + q0 * qrs;
+    const unsigned lane_off = (unsigned)(4 * h * qrs + n);
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int row = 8 * (r >> 2) + 4 * h + (r & 3);
-            dqp[row * D + 32 * db + n] = bf16_bits(dqacc[db][r]);
+            uint16_t* rowp = dqp + ((8 * (r >> 2) + (r & 3)) * qrs + 32 * db);
+            rowp[lane_off] = bf16_bits(dqacc[db][r]);
         }
 }
 
@@ -207,6 +211,7 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
 
     // ---- which tile, which walk
     int hk, nunits, list0 = 0, slot = -1;
+    int64_t qseq = 0;        // sequence of every query chunk this tile meets (indexed form)
     int64_t gz = 0;          // gathered: the single (z, j)
     int gj = 0;
     const uint16_t* kt;
@@ -219,6 +224,7 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
         const int64_t pair = (idx / seg_per) * NUM_XCD + blockIdx.x % NUM_XCD;
         if (pair >= p.N * p.Hkv) return;
         const int64_t nseq = pair / p.Hkv;
+        qseq = nseq;
         hk = (int)(pair % p.Hkv);
         const int seg_lo = ws.seg_base[nseq * p.C];
         const int seg_hi = nseq + 1 < p.N ? ws.seg_base[(nseq + 1) * p.C] : ws.nseg[0];
@@ -270,7 +276,7 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
         for (int r = 0; r < 16; ++r) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
 
     const float c = p.sm_scale * LOG2E;
-    const TileLoader<D, NT> loader(tid, D);
+    const TileLoader<D, NT> loader(tid, (int)p.q_rs);
 
     // unit u = (reference, query head of the group, 64-row query tile), tile fastest
     const int nqt = p.Q_CTX / 64;
@@ -293,7 +299,7 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
     auto issue_unit = [&](int u, int buf) -> float {
         int64_t z; int j, hq, qrow0;
         unit_coords(u, z, j, hq, qrow0);
-        const int64_t qoff = ((z * p.Hq + hq) * (int64_t)p.Q_CTX + qrow0) * D;
+        const int64_t qoff = q_base_n(p, qseq, z, hq) + qrow0 * (int)p.q_rs;
         const int64_t loffq = ((z * p.Hq + hq) * (int64_t)p.K + j) * p.Q_CTX + qrow0;
         unsigned char* nb = smem + buf * BUF;
         loader.issue(q + qoff, nb);
@@ -414,6 +420,7 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
 
     // ---- which tile, which walk
     int hk, nunits, list0 = 0, slot = -1;
+    int64_t qseq = 0;        // sequence of every query chunk this tile meets (indexed form)
     int64_t gz = 0;          // gathered: the single (z, j)
     int gj = 0;
     const uint16_t* kt;
@@ -426,6 +433,7 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
         const int64_t pair = (idx / seg_per) * NUM_XCD + blockIdx.x % NUM_XCD;
         if (pair >= p.N * p.Hkv) return;
         const int64_t nseq = pair / p.Hkv;
+        qseq = nseq;
         hk = (int)(pair % p.Hkv);
         const int seg_lo = ws.seg_base[nseq * p.C];
         const int seg_hi = nseq + 1 < p.N ? ws.seg_base[(nseq + 1) * p.C] : ws.nseg[0];
@@ -477,7 +485,7 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
         for (int r = 0; r < 16; ++r) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
 
     const float c = p.sm_scale * LOG2E;
-    const TileLoader<D, NT> loader(tid, D);
+    const TileLoader<D, NT> loader(tid, (int)p.q_rs);
 
     // unit u = (reference, query head of the group, 64-row query tile), tile fastest
     const int nqt = p.Q_CTX / 64;
@@ -504,7 +512,7 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
     auto issue_unit = [&](int u, int buf) -> float {
         int64_t z; int j, hq, qrow0;
         unit_coords(u, z, j, hq, qrow0);
-        const int64_t qoff = ((z * p.Hq + hq) * (int64_t)p.Q_CTX + qrow0) * D;
+        const int64_t qoff = q_base_n(p, qseq, z, hq) + qrow0 * (int)p.q_rs;
         loff_next = ((z * p.Hq + hq) * (int64_t)p.K + j) * p.Q_CTX + qrow0 + 32 * sub + 4 * h;
         unsigned char* nb = smem + buf * BUF;
         loader.issue(q + qoff, nb);
@@ -684,7 +692,7 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
         const int64_t blocks = (p.N * p.Hkv + NUM_XCD - 1) / NUM_XCD * NUM_XCD * seg_per;
         if (blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
         if (!(p.stages & GCA_STAGE_DKDV)) {
-        } else if (D == 64)
+        } else if constexpr (D == 64)
             hipLaunchKernelGGL((gca_bwd_dkdv2_mfma_kernel<D, true>), dim3((unsigned)blocks), dim3(128), 0, s, p,
                                (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
                                delta, dk, dv, ws, seg_per);
@@ -699,7 +707,7 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
         const int64_t blocks = p.Z * p.Hkv * p.K;
         if (blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
         if (!(p.stages & GCA_STAGE_DKDV)) {
-        } else if (D == 64)
+        } else if constexpr (D == 64)
             hipLaunchKernelGGL((gca_bwd_dkdv2_mfma_kernel<D, false>), dim3((unsigned)blocks), dim3(128), 0, s, p,
                                (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
                                delta, dk, dv, ws, seg_per0);

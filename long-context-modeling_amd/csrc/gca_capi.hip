@@ -15,8 +15,12 @@ int check_desc(const gca_desc* d, bool indexed) {
     if (!(d->sm_n >= 0.f)) return GCA_ERR_SHAPE;
     if (d->path != GCA_PATH_AUTO && d->path != GCA_PATH_GENERIC && d->path != GCA_PATH_MFMA) return GCA_ERR_SHAPE;
     if (d->stages < 0 || d->stages > 31) return GCA_ERR_SHAPE;
+    if (d->q_layout != GCA_Q_HEAD_MAJOR && d->q_layout != GCA_Q_TOKEN_MAJOR) return GCA_ERR_SHAPE;
+    if (d->q_skip < 0 || (d->q_skip > 0 && d->q_layout != GCA_Q_TOKEN_MAJOR)) return GCA_ERR_SHAPE;
     if (indexed) {
         if (d->N <= 0 || d->C <= 0 || d->Z % d->N != 0) return GCA_ERR_SHAPE;
+    } else if (d->q_layout != GCA_Q_HEAD_MAJOR) {
+        return GCA_ERR_UNSUPPORTED;
     }
     return GCA_OK;
 }
@@ -71,8 +75,9 @@ int gca_fwd(const gca_desc* desc, const void* q, const void* k, const void* v, c
 }
 
 size_t gca_bwd_workspace_bytes(const gca_desc* desc) {
-    if (check_desc(desc, false) != GCA_OK) return 0;
-    const bool indexed = desc->N > 0 && desc->C > 0 && desc->Z % desc->N == 0;
+    if (desc == nullptr) return 0;
+    const bool indexed = desc->N > 0 && desc->C > 0 && desc->Z > 0 && desc->Z % desc->N == 0;
+    if (check_desc(desc, indexed) != GCA_OK) return 0;
     return bwd_workspace_bytes(*desc, indexed);
 }
 

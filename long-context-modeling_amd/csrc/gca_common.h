@@ -38,6 +38,9 @@ struct Params {
     int64_t N, C, zpn;   // zpn = Z / N rows per sequence
     int32_t indexed;
     int32_t stages;      // gca_stage bitmask, never 0 here
+    // q / o / dO / dq addressing: element strides of a query chunk, a head and a row; q_skip leading
+    // chunks of every sequence are skipped (token-major form only)
+    int64_t q_zs, q_hs, q_rs, q_skip;
 };
 
 inline Params make_params(const gca_desc& d, bool indexed) {
@@ -49,6 +52,11 @@ inline Params make_params(const gca_desc& d, bool indexed) {
     p.zpn = indexed ? d.Z / d.N : d.Z;
     p.indexed = indexed ? 1 : 0;
     p.stages = d.stages == 0 ? 31 : d.stages;
+    if (d.q_layout == GCA_Q_TOKEN_MAJOR) {
+        p.q_rs = (int64_t)d.Hq * d.D; p.q_hs = d.D; p.q_zs = (int64_t)d.Q_CTX * d.Hq * d.D; p.q_skip = d.q_skip;
+    } else {
+        p.q_rs = d.D; p.q_hs = (int64_t)d.Q_CTX * d.D; p.q_zs = (int64_t)d.Hq * d.Q_CTX * d.D; p.q_skip = 0;
+    }
     return p;
 }
 
@@ -66,6 +74,15 @@ __device__ __forceinline__ const T* chunk_base_n(const Params& p, const T* base,
     }
     row_stride = p.D;
     return base + (((z * p.Hkv + hk) * p.K + j) * (int64_t)p.K_CTX) * p.D;
+}
+
+// Element offset of (row 0, dim 0) of query chunk z (of sequence n), head h in q / o / dO / dq;
+// consecutive rows are p.q_rs elements apart.
+__device__ __forceinline__ int64_t q_base_n(const Params& p, int64_t n, int64_t z, int h) {
+    return (z + (n + 1) * p.q_skip) * p.q_zs + h * p.q_hs;
+}
+__device__ __forceinline__ int64_t q_base(const Params& p, int64_t z, int h) {
+    return q_base_n(p, p.q_skip ? z / p.zpn : 0, z, h);
 }
 
 // Same, for callers that do not know the row's sequence n = z / zpn yet.

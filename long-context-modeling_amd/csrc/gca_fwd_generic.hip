@@ -37,7 +37,7 @@ gca_fwd_generic_kernel(Params p, const T* __restrict__ q, const T* __restrict__ 
 #pragma unroll
     for (int i = 0; i < DPT; ++i) { qreg[i] = 0.f; acc[i] = 0.f; }
     if (row_ok) {
-        const T* qp = q + ((z * p.Hq + h) * (int64_t)p.Q_CTX + row) * D + t * DPT;
+        const T* qp = q + q_base(p, z, h) + row * p.q_rs + t * DPT;
 #pragma unroll
         for (int i = 0; i < DPT; ++i) qreg[i] = to_f(qp[i]);
     }
@@ -104,7 +104,7 @@ gca_fwd_generic_kernel(Params p, const T* __restrict__ q, const T* __restrict__ 
             lse[((z * p.Hq + h) * (int64_t)p.K + j) * p.Q_CTX + row] = m + log2f(l);
     }
     if (row_ok) {
-        T* op = o + ((z * p.Hq + h) * (int64_t)p.Q_CTX + row) * D + t * DPT;
+        T* op = o + q_base(p, z, h) + row * p.q_rs + t * DPT;
 #pragma unroll
         for (int i = 0; i < DPT; ++i) op[i] = from_f<T>(acc[i]);
     }

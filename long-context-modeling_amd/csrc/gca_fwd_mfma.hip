@@ -61,10 +61,11 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
     const int q0 = qt * 64 + qb * 32;
 
     // Q as the B operand: lane holds row n, dims 16*ks + 8*h .. +7
+    const int qrs = (int)p.q_rs;               // row stride of q / o in elements (32-bit index math below)
     bf16x8 qB[KS];
     const bool row_ok = q0 + n < p.Q_CTX;      // false only in the last tile of a Q_CTX that is not a multiple of 64
     {
-        const uint16_t* qp = q + ((z * p.Hq + hq) * (int64_t)p.Q_CTX + q0 + n) * D + 8 * h;
+        const uint16_t* qp = q + q_base_n(p, nseq, z, hq) + (q0 + n) * qrs + 8 * h;
         const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) qB[ks] = row_ok ? *reinterpret_cast<const bf16x8*>(qp + 16 * ks) : zero8;
@@ -176,14 +177,17 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
     }
 
     // ---- store O: register r of block db is row 8*(r/4) + 4*h + r%4, column 32*db + n
-    uint16_t* op = o + ((z * p.Hq + hq) * (int64_t)p.Q_CTX + q0) * D;
+    //      = a wavefront-uniform base per (r, db) plus one 32-bit lane offset
+    uint16_t* op = o + q_base_n(p, nseq, z, hq) + q0 * qrs;
+    const unsigned lane_off = (unsigned)(4 * h * qrs + n);
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int row = 8 * (r >> 2) + 4 * h + (r & 3);
             const __bf16 ob = (__bf16)oacc[db][r];
-            if (q0 + row < p.Q_CTX) op[row * D + 32 * db + n] = __builtin_bit_cast(uint16_t, ob);
+            uint16_t* rowp = op + ((8 * (r >> 2) + (r & 3)) * qrs + 32 * db);
+            if (q0 + row < p.Q_CTX) rowp[lane_off] = __builtin_bit_cast(uint16_t, ob);
         }
 }
 

@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libgca_hip.so")
 
 GCA_F32, GCA_BF16 = 0, 1
 GCA_PATH_AUTO, GCA_PATH_GENERIC, GCA_PATH_MFMA = 0, 1, 2
+GCA_Q_HEAD_MAJOR, GCA_Q_TOKEN_MAJOR = 0, 1
 GCA_OK = 0
 
 SYMBOLS = (
@@ -33,6 +34,7 @@ class GcaDesc(ctypes.Structure):
         ("sm_scale", ctypes.c_float), ("sm_n", ctypes.c_float),
         ("path", ctypes.c_int32), ("stages", ctypes.c_int32),
         ("N", ctypes.c_int64), ("C", ctypes.c_int64),
+        ("q_layout", ctypes.c_int32), ("q_skip", ctypes.c_int32),
     ]
 
 

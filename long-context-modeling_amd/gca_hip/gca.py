@@ -10,6 +10,8 @@ and adds the cache-indexed form that skips the K-times-larger gather copies of
 model/DRT.py:193-200 and :320-332:
 
 * ``attention_indexed(q, k_cache, v_cache, indices, weights, sm_scale, sm_n)``.
+* ``attention_tokens(q_tok, k_cache, v_cache, indices, weights, num_heads, sm_n)``: the same on the
+  projection's own (N, C, S, Hq*d) layout, without the permute copies of model/DRT.py:366-378 and :384.
 
 Shapes: q (Z, Hq, Q_CTX, d); k, v (Z, Hkv, K, K_CTX, d); weights (Z, K) shared by all heads
 (reference :118); output (Z, Hq, Q_CTX, d) in q's dtype.  k_cache, v_cache (N, C, K_CTX, Hkv*d),
@@ -57,11 +59,18 @@ def _check_inputs(q, k, v, weights):
     assert weights.dtype in _DT, f"unsupported weights dtype {weights.dtype}"
 
 
-def _desc(q, K, K_CTX, Hkv, weights, sm_scale, sm_n, path=None, N=0, C=0):
-    Z, Hq, Q_CTX, D = q.shape
+def _desc(q, K, K_CTX, Hkv, weights, sm_scale, sm_n, path=None, N=0, C=0, token_shape=None):
+    """``token_shape`` = (Z, Hq, Q_CTX, D, q_skip) describes a token-major q (N, Z/N + q_skip, Q_CTX, Hq*D)."""
+    if token_shape is None:
+        Z, Hq, Q_CTX, D = q.shape
+        layout, skip = _lib.GCA_Q_HEAD_MAJOR, 0
+    else:
+        Z, Hq, Q_CTX, D, skip = token_shape
+        layout = _lib.GCA_Q_TOKEN_MAJOR
     return _lib.GcaDesc(
         dtype=_DT[q.dtype], w_dtype=_DT[weights.dtype], Z=Z, Hq=Hq, Hkv=Hkv, K=K, Q_CTX=Q_CTX, K_CTX=K_CTX, D=D,
-        sm_scale=float(sm_scale), sm_n=float(sm_n), path=_PATHS[path or kernel_path], stages=0, N=N, C=C)
+        sm_scale=float(sm_scale), sm_n=float(sm_n), path=_PATHS[path or kernel_path], stages=0, N=N, C=C,
+        q_layout=layout, q_skip=skip)
 
 
 def _forward(q, k, v, weights, sm_scale, sm_n, want_lse, path=None):
@@ -195,3 +204,79 @@ def gca_kv_cache_indexed(q, k_cache, v_cache, indices, weights, sm_scale, sm_n=0
                                             _ptr(weights), _ptr(o), ctypes.c_void_p(0), _stream(q.device))
         _lib.check(rc, "gca_fwd_indexed")
         return o
+
+
+# ------------------------------------------------------------------------------- token-major form
+
+class _AttentionTokens(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q_tok, k_cache, v_cache, indices, weights, num_heads, sm_scale, sm_n, want_grad):
+        N, C, S, HD = q_tok.shape
+        D = HD // num_heads
+        Nc, Cc, K_CTX, Dm = k_cache.shape
+        kk = indices.shape[-1]
+        Z = N * (C - 1)
+        idx = indices[:, :-1].reshape(Z, kk).contiguous()        # row c feeds query chunk c+1 (model/DRT.py:629)
+        w = weights[:, :-1].reshape(Z, kk).contiguous()
+        o = torch.empty_like(q_tok)
+        o[:, 0].zero_()                                          # chunk 0 retrieves nothing (model/DRT.py:387-394)
+        lse = torch.empty((Z, num_heads, kk, S), device=q_tok.device, dtype=torch.float32) if want_grad else None
+        desc = _desc(q_tok, kk, K_CTX, Dm // D, w, sm_scale, sm_n, N=Nc, C=Cc, token_shape=(Z, num_heads, S, D, 1))
+        with torch.cuda.device(q_tok.device):
+            rc = _lib.lib().gca_fwd_indexed(ctypes.byref(desc), _ptr(q_tok), _ptr(k_cache), _ptr(v_cache), _ptr(idx),
+                                            _ptr(w), _ptr(o), _ptr(lse), _stream(q_tok.device))
+        _lib.check(rc, "gca_fwd_indexed")
+        if want_grad:
+            ctx.save_for_backward(q_tok, k_cache, v_cache, idx, w, lse)
+            ctx.args = (num_heads, float(sm_scale), float(sm_n), weights.dtype, weights.shape)
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q_tok, k_cache, v_cache, idx, w, lse = ctx.saved_tensors
+        num_heads, sm_scale, sm_n, w_dtype, w_shape = ctx.args
+        do = do.contiguous()
+        N, C, S, HD = q_tok.shape
+        D = HD // num_heads
+        Nc, Cc, K_CTX, Dm = k_cache.shape
+        Z, kk = idx.shape
+        dq = torch.empty_like(q_tok)
+        dq[:, 0].zero_()
+        dkc, dvc = torch.empty_like(k_cache), torch.empty_like(v_cache)
+        dw = torch.zeros(w_shape, device=q_tok.device, dtype=torch.float32)      # last retrieval row: unused, gradient 0
+        dwz = torch.empty((Z, kk), device=q_tok.device, dtype=torch.float32)
+        desc = _desc(q_tok, kk, K_CTX, Dm // D, w, sm_scale, sm_n, N=Nc, C=Cc, token_shape=(Z, num_heads, S, D, 1))
+        with torch.cuda.device(q_tok.device):
+            L = _lib.lib()
+            nbytes = L.gca_bwd_workspace_bytes(ctypes.byref(desc))
+            ws = torch.empty(nbytes // 4, device=q_tok.device, dtype=torch.float32)
+            rc = L.gca_bwd_indexed(ctypes.byref(desc), _ptr(q_tok), _ptr(k_cache), _ptr(v_cache), _ptr(idx), _ptr(w),
+                                   _ptr(do), _ptr(lse), _ptr(dq), _ptr(dkc), _ptr(dvc), _ptr(dwz), _ptr(ws), nbytes,
+                                   _stream(q_tok.device))
+        _lib.check(rc, "gca_bwd_indexed")
+        dw[:, :-1] = dwz.view(N, C - 1, kk)
+        return dq, dkc, dvc, None, dw.to(w_dtype), None, None, None, None
+
+
+def attention_tokens(q_tok, k_cache, v_cache, indices, weights, num_heads, sm_n=0.0, sm_scale=None):
+    """One GCA layer on the layouts the model already has (autograd-aware).
+
+    q_tok (N, C, S, Hq*d): the query projection of every chunk, as ``q_proj`` wrote it; k_cache, v_cache
+    (N, C', S, Hkv*d) (C' >= C: a store with spare capacity is fine); indices, weights (N, C, kk) as the
+    retrieval returns them: row c feeds chunk c+1, the last row is not used (model/DRT.py:629-637).
+    Returns (N, C, S, Hq*d) with chunk 0 zero, ready for ``o_proj``; replaces model/DRT.py:366-384 without
+    the two permute copies.  ``sm_scale`` defaults to 1/sqrt(d) (model/DRT.py:380).
+    """
+    assert q_tok.is_cuda and q_tok.dim() == 4 and q_tok.is_contiguous() and q_tok.dtype in _DT
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape == v_cache.shape and k_cache.dim() == 4
+    assert k_cache.dtype == q_tok.dtype and v_cache.dtype == q_tok.dtype and weights.dtype in _DT
+    N, C, S, HD = q_tok.shape
+    assert HD % num_heads == 0 and (HD // num_heads) in _HEAD_DIMS, f'current head dim: {HD // num_heads}'
+    D = HD // num_heads
+    assert k_cache.shape[0] == N and k_cache.shape[3] % D == 0 and num_heads % (k_cache.shape[3] // D) == 0
+    assert indices.dtype == torch.int64 and indices.shape == weights.shape and indices.shape[:2] == (N, C)
+    if C < 2 or indices.shape[-1] == 0:
+        return torch.zeros_like(q_tok)                            # nothing to retrieve (model/DRT.py:359-364)
+    sm_scale = D ** -0.5 if sm_scale is None else sm_scale
+    want_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (q_tok, k_cache, v_cache, weights))
+    return _AttentionTokens.apply(q_tok, k_cache, v_cache, indices, weights, num_heads, sm_scale, sm_n, want_grad)

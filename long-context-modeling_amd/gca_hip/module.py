@@ -1,0 +1,56 @@
+"""The GCA sub-layer as a module: RMSNorm -> q_proj -> chunk attention -> o_proj.
+
+Mirrors ``TritonGroupCrossAttention`` of the reference (model/DRT.py:304-398) with the same parameters
+(``pre_norm``, ``q_proj``, ``o_proj``) so a checkpoint's state dict loads, and the same results, but the
+attention runs on the projection's own (N, C, S, Hq*d) layout: the reference's two rearrange + contiguous
+copies around the kernel (DRT.py:366-378, :384) and the zero-filled output copy (DRT.py:387-394) are gone,
+and because the kernels read retrieved chunks from the cache by index, the one retrieval of a layer group
+(DRT.py:816-822) serves all its layers with no gathered copy at all.
+"""
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from .gca import attention_tokens
+
+
+class GroupCrossAttention(nn.Module):
+    def __init__(self, hidden_size, num_heads, enc_chunk_size=64, chunk_topk=8, rms_norm_eps=1e-6,
+                 attention_bias=False, enable_softmax_one=False):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.head_dim = hidden_size // num_heads
+        self.enc_chunk_size = enc_chunk_size
+        self.topK = chunk_topk
+        self.pre_norm = nn.RMSNorm(hidden_size, eps=rms_norm_eps)
+        self.q_proj = nn.Linear(hidden_size, num_heads * self.head_dim, bias=attention_bias)
+        self.o_proj = nn.Linear(hidden_size, num_heads * self.head_dim, bias=attention_bias)
+        self.sm_n = 1.0 if enable_softmax_one else 0.0            # DRT.py:318-319
+
+    def forward(self, hidden_states, chunk_kvs, indices, weights):
+        """hidden_states (N, C, S, dim); ``chunk_kvs`` a ChunkKVManager (or a (k_store, v_store) pair);
+        indices, weights (N, C, kk) from the group's retrieval.  Returns (N, C*S, dim), chunk 0 zero
+        (DRT.py:345-398 with chunk_size > 1)."""
+        N, C, S, dim = hidden_states.shape
+        if weights.shape[0] * weights.shape[1] == 0:              # DRT.py:359-364
+            return torch.zeros((N, C * S, dim), device=hidden_states.device, dtype=hidden_states.dtype)
+        k_store, v_store = (chunk_kvs.k_store, chunk_kvs.v_store) if hasattr(chunk_kvs, "k_store") else chunk_kvs
+        q = self.q_proj(self.pre_norm(hidden_states))             # (N, C, S, Hq*d), read in place by the kernel
+        vals = attention_tokens(q.contiguous(), k_store, v_store, indices, weights, self.num_heads, self.sm_n)
+        o = self.o_proj(vals)                                     # chunk 0 of vals is zero
+        if self.o_proj.bias is not None:
+            keep = torch.ones((1, C, 1, 1), device=o.device, dtype=o.dtype)
+            keep[:, 0] = 0
+            o = o * keep                                          # the reference leaves chunk 0 at exactly zero
+        return o.view(N, C * S, dim)
+
+    @torch.no_grad()
+    def decode(self, hidden_states, chunk_kvs, group_idx=0):
+        """hidden_states (N, Q, dim), Q = 1 or 2 tokens being generated; uses the group's retrieval state
+        (DRT.py:345-398 with chunk_size == 1, :825-831).  Returns (N, Q, dim)."""
+        N, Q, dim = hidden_states.shape
+        q = self.q_proj(self.pre_norm(hidden_states)).view(N, Q, self.num_heads, self.head_dim)
+        vals = chunk_kvs.decode_attention(q.transpose(1, 2).contiguous(), group_idx, self.sm_n)   # (N, Hq, Q, d)
+        return self.o_proj(vals.transpose(1, 2).reshape(N, Q, self.num_heads * self.head_dim))

@@ -253,3 +253,31 @@ def gca_layer(q_all, chunk_k, chunk_v, lmk_q, lmk_k, chunk_topk: int, num_kv_hea
     out = torch.zeros_like(q_all)
     out[:, 1:] = o.reshape(N, C - 1, Hq, S, d)
     return out, indices, weights
+
+
+# --------------------------------------------------------------------------- the sub-layer around the kernel
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """x / sqrt(mean(x^2) + eps) * weight over the last dim (the RMSNorm of model/DRT.py:314, :353)."""
+    return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * weight
+
+
+def gca_module_forward(hidden, chunk_k, chunk_v, indices, weights, norm_w, eps, wq, bq, wo, bo, num_heads: int,
+                       num_kv_heads: int, sm_n: float = 0.0):
+    """TritonGroupCrossAttention.forward for chunk_size > 1, step by step (model/DRT.py:345-398):
+    pre_norm -> q_proj -> 'N D S (h d) -> N D h S d' -> drop chunk 0 -> '(N D) h S d' -> kernel with
+    sm_scale = 1/sqrt(d) -> '(N D) h S d -> N (D S) (h d)' -> o_proj -> zero-filled result whose last
+    (C-1)*S rows are the output.  hidden (N, C, S, dim); indices/weights (N, C, kk) from the retrieval."""
+    N, C, S, dim = hidden.shape
+    d = dim // num_heads
+    x = rms_norm(hidden, norm_w, eps)
+    q = F.linear(x, wq, bq)                                             # (N, C, S, h*d)
+    q = q.reshape(N, C, S, num_heads, d).permute(0, 1, 3, 2, 4)         # N D h S d
+    q = q[:, 1:].reshape(N * (C - 1), num_heads, S, d)                  # model/DRT.py:369-372
+    k, v, w = gather_chunks(chunk_k, chunk_v, indices, weights, num_kv_heads)
+    vals = gca_forward(q, k, v, w, 1.0 / math.sqrt(d), sm_n)            # ((N D), h, S, d)
+    vals = vals.reshape(N, C - 1, num_heads, S, d).permute(0, 1, 3, 2, 4).reshape(N, (C - 1) * S, num_heads * d)
+    o = F.linear(vals, wo, bo)
+    ret = torch.zeros((N, C * S, dim), dtype=o.dtype)
+    ret[:, -o.shape[1]:, :] = o                                         # model/DRT.py:387-394
+    return ret

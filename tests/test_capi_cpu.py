@@ -28,7 +28,8 @@ def test_library_exports_every_declared_symbol():
 
 def test_struct_layout_matches_header():
     # offsets implied by the C declaration order with natural alignment
-    assert ctypes.sizeof(_lib.GcaDesc) == 72 and _lib.GcaDesc.Z.offset == 8 and _lib.GcaDesc.N.offset == 56
+    assert ctypes.sizeof(_lib.GcaDesc) == 80 and _lib.GcaDesc.Z.offset == 8 and _lib.GcaDesc.N.offset == 56
+    assert _lib.GcaDesc.q_layout.offset == 72 and _lib.GcaDesc.q_skip.offset == 76
     assert ctypes.sizeof(_lib.LmkDesc) == 48 and _lib.LmkDesc.E.offset == 24 and _lib.LmkDesc.hidden_size.offset == 40
 
 
@@ -79,6 +80,22 @@ def test_missing_library_is_an_error(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libgca_hip.so")
     with pytest.raises(RuntimeError):
         _lib.lib()
+
+
+def test_q_layout_validation():
+    """Token-major q is an indexed-entry feature; bad layout values are refused (no GPU needed)."""
+    import ctypes
+    from gca_hip import _lib
+    L = _lib.lib()
+    one = ctypes.c_void_p(16)
+    base = dict(dtype=1, w_dtype=0, Z=4, Hq=2, Hkv=2, K=2, Q_CTX=64, K_CTX=64, D=64, sm_scale=0.125, sm_n=0.0,
+                path=0, stages=0, N=2, C=3)
+    d = _lib.GcaDesc(**base, q_layout=1, q_skip=1)
+    assert L.gca_fwd(ctypes.byref(d), one, one, one, one, one, None, None) == 6          # gathered form: head-major only
+    d = _lib.GcaDesc(**base, q_layout=2, q_skip=0)
+    assert L.gca_fwd_indexed(ctypes.byref(d), one, one, one, one, one, one, None, None) == 2
+    d = _lib.GcaDesc(**base, q_layout=0, q_skip=1)
+    assert L.gca_fwd_indexed(ctypes.byref(d), one, one, one, one, one, one, None, None) == 2
 
 
 def test_chunk_cache_desc_layout_and_validation():

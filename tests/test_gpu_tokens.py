@@ -1,0 +1,143 @@
+"""GPU parity of the token-major entry (q, o, dO, dq in the projection's own (N, C, S, Hq*d) layout) and of
+the sub-layer module built on it, against the CPU oracle and against the head-major entry, through the C ABI.
+
+Tolerances as everywhere: 1e-5 relative fp32, 2e-2 bf16 (max |err| / max |ref| per tensor); the two layouts
+run the same kernels on the same numbers, so their results must be bit-identical."""
+import math
+
+import pytest
+import torch
+
+from helpers import gen, rel_err
+from oracle import gca_oracle as orc
+
+pytestmark = pytest.mark.gpu
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
+
+
+def _inputs(N, C, Hq, Hkv, S, d, topk, dtype, seed):
+    q_tok = gen((N, C, S, Hq * d), seed, 0.5, dtype)
+    ck = gen((N, C, S, Hkv * d), seed + 1, 0.5, dtype)
+    cv = gen((N, C, S, Hkv * d), seed + 2, 0.5, dtype)
+    lq, lk = gen((N, C, 32), seed + 3, 1.0, torch.float32), gen((N, C, 32), seed + 4, 1.0, torch.float32)
+    _, idx, w = orc.retrieve(lq, lk, topk)
+    do = gen((N, C, S, Hq * d), seed + 5, 1.0, dtype)
+    return q_tok, ck, cv, idx, w, do
+
+
+def _head_major(t, Hq):
+    N, C, S, HD = t.shape
+    return t.view(N, C, S, Hq, HD // Hq).permute(0, 1, 3, 2, 4)[:, 1:].reshape(N * (C - 1), Hq, S, HD // Hq).contiguous()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [
+    # N, C, Hq, Hkv, S, d, topk
+    (2, 5, 4, 4, 64, 64, 3),
+    (3, 4, 8, 2, 64, 128, 2),      # 4 query heads per kv head, d=128
+    (1, 9, 2, 1, 64, 64, 4),
+    (2, 3, 4, 2, 128, 64, 2),      # two 64-row tiles per chunk
+    (2, 4, 6, 3, 24, 32, 2),       # generic kernels in both dtypes
+])
+def test_token_major_equals_head_major_and_oracle(shape, dtype):
+    import gca_hip
+    N, C, Hq, Hkv, S, d, topk = shape
+    q_tok, ck, cv, idx, w, do = _inputs(N, C, Hq, Hkv, S, d, topk, dtype, seed=130)
+    kk = idx.shape[-1]
+    # token-major
+    qg, kg, vg, wg = [t.cuda().requires_grad_() for t in (q_tok, ck, cv, w)]
+    out = gca_hip.attention_tokens(qg, kg, vg, idx.cuda(), wg, Hq, sm_n=1.0)
+    out.backward(do.cuda())
+    assert out.shape == q_tok.shape and out[:, 0].abs().max() == 0 and qg.grad[:, 0].abs().max() == 0
+    assert wg.grad[:, -1].abs().max() == 0
+    # head-major on the same numbers
+    q2, k2, v2, w2 = [t.cuda().requires_grad_() for t in (_head_major(q_tok, Hq), ck, cv, w[:, :-1].reshape(-1, kk))]
+    o2 = gca_hip.attention_indexed(q2, k2, v2, idx[:, :-1].reshape(-1, kk).contiguous().cuda(), w2, 1 / math.sqrt(d), 1.0)
+    o2.backward(_head_major(do, Hq).cuda())
+    assert torch.equal(_head_major(out.detach().cpu(), Hq), o2.detach().cpu())
+    assert torch.equal(_head_major(qg.grad.cpu(), Hq), q2.grad.cpu())
+    assert torch.equal(kg.grad, k2.grad) and torch.equal(vg.grad, v2.grad)
+    assert torch.equal(wg.grad[:, :-1].reshape(-1, kk), w2.grad)
+    # oracle (float64 on the rounded inputs)
+    qo, ko, vo, wo = [t.double().requires_grad_() for t in (_head_major(q_tok, Hq), ck, cv, w)]
+    kgat, vgat, wgat = orc.gather_chunks(ko, vo, idx, wo, Hkv)
+    oo = orc.gca_forward(qo, kgat, vgat, wgat, 1 / math.sqrt(d), 1.0)
+    oo.backward(_head_major(do, Hq).double())
+    tol = TOL[dtype]
+    assert rel_err(o2, oo) < tol and rel_err(q2.grad, qo.grad) < tol
+    assert rel_err(kg.grad, ko.grad) < tol and rel_err(vg.grad, vo.grad) < tol
+    assert rel_err(wg.grad, wo.grad) < (tol if dtype == torch.float32 else 3e-2)
+
+
+def test_token_major_inference_and_capacity_store():
+    """No-grad call (no LSE), caches that are stores with spare capacity."""
+    import gca_hip
+    N, C, Hq, Hkv, S, d, topk = 2, 6, 4, 2, 64, 64, 3
+    q_tok, ck, cv, idx, w, _ = _inputs(N, C, Hq, Hkv, S, d, topk, torch.bfloat16, seed=150)
+    m = gca_hip.ChunkKVManager(capacity=16)
+    with torch.no_grad():
+        m.append(ck.cuda(), cv.cuda(), torch.zeros(N, C, 8, device="cuda", dtype=torch.bfloat16))
+        a = gca_hip.attention_tokens(q_tok.cuda(), m.k_store, m.v_store, idx.cuda(), w.cuda(), Hq, sm_n=0.0)
+    b = gca_hip.attention_tokens(q_tok.cuda(), ck.cuda(), cv.cuda(), idx.cuda(), w.cuda(), Hq, sm_n=0.0)
+    assert torch.equal(a, b)
+    one = gca_hip.attention_tokens(q_tok[:, :1].contiguous().cuda(), ck.cuda(), cv.cuda(), idx[:, :1].cuda(), w[:, :1].cuda(), Hq)
+    assert one.abs().max() == 0                                   # a single chunk retrieves nothing
+
+
+@pytest.mark.parametrize("dtype,bias", [(torch.float32, True), (torch.float32, False), (torch.bfloat16, False)])
+def test_module_matches_oracle(dtype, bias):
+    """GroupCrossAttention (norm, projections, token-major kernels) == the oracle's step-by-step restatement of
+    the reference module, values and gradients (hidden, projections, norm weight, caches, retrieval weights)."""
+    import gca_hip
+    N, C, S, H, Hkv, d, topk = 2, 5, 64, 4, 2, 64, 3
+    dim = H * d
+    torch.manual_seed(5)
+    mod = gca_hip.GroupCrossAttention(dim, H, 64, topk, 1e-6, attention_bias=bias, enable_softmax_one=True)
+    with torch.no_grad():
+        mod.pre_norm.weight.copy_(1 + 0.1 * torch.randn(dim))
+    mod = mod.to(dtype).cuda()
+    hidden = gen((N, C, S, dim), 160, 1.0, dtype)
+    ck, cv = gen((N, C, S, Hkv * d), 161, 0.5, dtype), gen((N, C, S, Hkv * d), 162, 0.5, dtype)
+    lq, lk = gen((N, C, 32), 163), gen((N, C, 32), 164)
+    _, idx, w = orc.retrieve(lq, lk, topk)
+    dret = gen((N, C * S, dim), 165, 1.0, dtype)
+    hg, kg, vg, wg = [t.cuda().requires_grad_() for t in (hidden, ck, cv, w)]
+    ret = mod(hg, (kg, vg), idx.cuda(), wg)
+    ret.backward(dret.cuda())
+    # oracle in float64 on the module's (rounded) parameters
+    P = {n: p.detach().double().cpu().requires_grad_() for n, p in mod.named_parameters()}
+    ho, ko, vo, wo = [t.double().requires_grad_() for t in (hidden, ck, cv, w)]
+    ref = orc.gca_module_forward(ho, ko, vo, idx, wo, P["pre_norm.weight"], 1e-6, P["q_proj.weight"], P.get("q_proj.bias"),
+                                 P["o_proj.weight"], P.get("o_proj.bias"), H, Hkv, sm_n=1.0)
+    ref.backward(dret.double())
+    tol = 2e-4 if dtype == torch.float32 else 3e-2        # fp32: two library GEMMs of depth 256 around the kernel
+    assert ret.shape == ref.shape and ret[:, :S].abs().max() == 0
+    assert rel_err(ret, ref) < tol
+    assert rel_err(hg.grad, ho.grad) < tol and rel_err(kg.grad, ko.grad) < tol and rel_err(vg.grad, vo.grad) < tol
+    assert rel_err(wg.grad, wo.grad) < tol
+    for n, p in mod.named_parameters():
+        assert rel_err(p.grad, P[n].grad) < tol, n
+
+
+def test_module_decode_matches_batch_form():
+    """Module.decode on a ChunkKVManager state == the rows the batch forward produces for the same positions."""
+    import gca_hip
+    N, C, S, H, Hkv, d, topk = 2, 4, 64, 4, 2, 64, 2
+    dim = H * d
+    torch.manual_seed(6)
+    mod = gca_hip.GroupCrossAttention(dim, H, 64, topk, 1e-6, enable_softmax_one=True).to(torch.bfloat16).cuda()
+    hidden = gen((N, C, S, dim), 170, 1.0, torch.bfloat16).cuda()
+    ck, cv = gen((N, C, S, Hkv * d), 171, 0.5, torch.bfloat16).cuda(), gen((N, C, S, Hkv * d), 172, 0.5, torch.bfloat16).cuda()
+    lq, lk = gen((N, C, 64), 173, 1.0, torch.bfloat16).cuda(), gen((N, C, 64), 174, 1.0, torch.bfloat16).cuda()
+    with torch.no_grad():
+        m = gca_hip.ChunkKVManager()
+        m.append(ck[:, :C - 1], cv[:, :C - 1], lk[:, :C - 1])
+        idx, w = m.batch_retrieval(lq[:, :C - 1], topk, 0, use_cache=True)      # state = row C-2 -> feeds chunk C-1
+        full_m = gca_hip.ChunkKVManager()
+        full_m.append(ck, cv, lk)
+        idx_full, w_full = full_m.batch_retrieval(lq, topk)
+        assert torch.equal(idx_full[:, :C - 1], idx)
+        full = mod(hidden, full_m, idx_full, w_full).view(N, C, S, dim)
+        for s0, n in ((0, 1), (1, 2), (62, 2)):
+            step = mod.decode(hidden[:, C - 1, s0:s0 + n], m, 0)
+            assert rel_err(step, full[:, C - 1, s0:s0 + n]) < 2e-2

@@ -305,3 +305,46 @@ def test_cache_oracle_vs_loops():
     assert torch.equal(z[:, :, :-1], x[:, :, :S - 1]) and z[:, :, -1].abs().max() == 0
     assert torch.equal(co.landmark_row(x, "drop"), x[:, :, :S])
     assert co.landmark_row(x, "keep") is x
+
+
+# ----------------------------------------------------------------------------- the sub-layer around the kernel
+
+def test_rms_norm_vs_library():
+    x, w = _rand(3, 5, 16, seed=70), _rand(16, seed=71)
+    assert (orc.rms_norm(x, w, 1e-6) - F.rms_norm(x, (16,), w, 1e-6)).abs().max().item() < 1e-12
+
+
+def test_module_forward_vs_loops():
+    """The module's layout conventions against per-position python loops: output row (n, c*S + s) is
+    o_proj of the heads' attention outputs side by side, chunk 0 is zero, chunk c uses retrieval row c-1."""
+    N, C, S, H, Hkv, d, topk = 2, 4, 3, 4, 2, 16, 2
+    dim = H * d
+    hidden = _rand(N, C, S, dim, seed=72)
+    ck, cv = _rand(N, C, S, Hkv * d, seed=73, scale=0.5), _rand(N, C, S, Hkv * d, seed=74, scale=0.5)
+    lq, lk = _rand(N, C, 8, seed=75), _rand(N, C, 8, seed=76)
+    nw, wq, bq, wo, bo = _rand(dim, seed=77), _rand(dim, dim, seed=78, scale=0.2), _rand(dim, seed=79), \
+        _rand(dim, dim, seed=80, scale=0.2), _rand(dim, seed=81)
+    _, idx, w = orc.retrieve(lq, lk, topk)
+    got = orc.gca_module_forward(hidden, ck, cv, idx, w.double(), nw, 1e-6, wq, bq, wo, bo, H, Hkv, sm_n=1.0)
+    assert got.shape == (N, C * S, dim) and got[:, :S].abs().max() == 0
+    for n in range(N):
+        for c in range(1, C):
+            for s in range(S):
+                x = hidden[n, c, s]
+                x = x / math.sqrt((x * x).mean().item() + 1e-6) * nw
+                qrow = wq @ x + bq
+                heads = []
+                for h in range(H):
+                    qh = qrow[h * d:(h + 1) * d]
+                    hk = h // (H // Hkv)
+                    acc = torch.zeros(d, dtype=torch.float64)
+                    for j in range(idx.shape[-1]):
+                        e = idx[n, c - 1, j].item()
+                        kk_ = ck[n, e, :, hk * d:(hk + 1) * d]
+                        vv_ = cv[n, e, :, hk * d:(hk + 1) * d]
+                        sc = (kk_ @ qh) / math.sqrt(d)
+                        p = torch.exp(sc) / (1.0 + torch.exp(sc).sum())
+                        acc += w[n, c - 1, j].double() * (p @ vv_)
+                    heads.append(acc)
+                ref = wo @ torch.cat(heads) + bo
+                assert (got[n, c * S + s] - ref).abs().max().item() < 1e-9
