@@ -1,0 +1,70 @@
+"""Edge cases of the indexed kernels on the GPU, against the CPU oracle, through the C ABI: odd and large
+slot counts, one slot, several sequences, chunk ids outside the cache (clamped like a safe gather), a single
+query chunk, rows whose slots all carry weight zero.  Tolerances: 1e-5 relative fp32, 2e-2 bf16."""
+import pytest
+import torch
+
+from helpers import gen, rel_err
+from oracle import gca_oracle as orc
+
+pytestmark = pytest.mark.gpu
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
+
+
+def _case(N, C, Hq, Hkv, S, d, K, dtype, seed, idx=None, w=None):
+    import gca_hip
+    ck = gen((N, C, S, Hkv * d), seed, 0.5, dtype)
+    cv = gen((N, C, S, Hkv * d), seed + 1, 0.5, dtype)
+    g = torch.Generator().manual_seed(seed + 2)
+    Z = N * (C - 1)
+    if idx is None:
+        idx = torch.randint(0, C, (Z, K), generator=g)
+    if w is None:
+        w = torch.softmax(torch.rand(Z, K, generator=g), -1)
+    q = gen((Z, Hq, S, d), seed + 3, 0.5, dtype)
+    do = gen((Z, Hq, S, d), seed + 4, 1.0, dtype)
+    # oracle on the clamped ids: gather -> forward -> autograd scatters the chunk gradients back
+    cl = idx.clamp(0, C - 1)
+    ck64, cv64, q64, w64 = [t.double().requires_grad_() for t in (ck, cv, q, w)]
+    G = Hkv
+    b = torch.arange(N).repeat_interleave(C - 1).unsqueeze(1)
+    kg = ck64[b, cl].reshape(Z, K, S, G, d).permute(0, 3, 1, 2, 4)
+    vg = cv64[b, cl].reshape(Z, K, S, G, d).permute(0, 3, 1, 2, 4)
+    o_ref = orc.gca_forward(q64, kg, vg, w64, d ** -0.5, 1.0)
+    o_ref.backward(do.double())
+    qd, ckd, cvd, wd = [t.cuda().requires_grad_() for t in (q, ck, cv, w)]
+    o = gca_hip.attention_indexed(qd, ckd, cvd, idx.cuda(), wd, d ** -0.5, 1.0)
+    o.backward(do.cuda())
+    tol = TOL[dtype]
+    for name, a, r in (("o", o, o_ref), ("dq", qd.grad, q64.grad), ("dk", ckd.grad, ck64.grad),
+                       ("dv", cvd.grad, cv64.grad), ("dw", wd.grad, w64.grad)):
+        assert torch.isfinite(a.float()).all(), name
+        assert rel_err(a, r) <= (tol if name != "dw" or dtype == torch.float32 else 3e-2), name
+    return o, qd.grad, ckd.grad, cvd.grad, wd.grad
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("N,C,Hq,Hkv,K", [(1, 5, 2, 2, 1), (3, 4, 4, 2, 7), (1, 3, 2, 1, 33), (2, 2, 6, 3, 5), (1, 80, 2, 2, 70)])
+def test_slot_counts_and_sequences(N, C, Hq, Hkv, K, dtype):
+    _case(N, C, Hq, Hkv, 64, 64, K, dtype, seed=300 + K)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_ids_outside_the_cache_are_clamped(dtype):
+    N, C, K = 2, 6, 4
+    g = torch.Generator().manual_seed(7)
+    idx = torch.randint(-3, C + 3, (N * (C - 1), K), generator=g)
+    idx[0, 0], idx[1, 1] = -(1 << 40), 1 << 40
+    _case(N, C, 4, 2, 64, 64, K, dtype, seed=320, idx=idx)
+
+
+def test_rows_with_no_weight_and_unretrieved_chunks():
+    N, C, K = 2, 7, 3
+    Z = N * (C - 1)
+    g = torch.Generator().manual_seed(9)
+    idx = torch.randint(0, 2, (Z, K), generator=g)             # only chunks 0 and 1 are ever retrieved
+    w = torch.softmax(torch.rand(Z, K, generator=g), -1)
+    w[::2] = 0                                                  # every other row has nothing retrieved
+    o, dq, dk, dv, dw = _case(N, C, 4, 4, 64, 64, K, torch.bfloat16, seed=330, idx=idx, w=w)
+    assert o[::2].abs().max() == 0 and dq[::2].abs().max() == 0
+    assert dk[:, 2:].abs().max() == 0 and dv[:, 2:].abs().max() == 0
