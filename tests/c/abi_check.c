@@ -1,0 +1,31 @@
+/* Plain C99 client of libgca_hip.so: proves that include/gca_hip.h is valid C, that the struct sizes the
+ * Python binding assumes are the compiler's, and that argument validation answers before any GPU work. */
+#include <stdio.h>
+#include <string.h>
+#include "gca_hip.h"
+
+int main(void) {
+    gca_desc d;
+    lmk_desc l;
+    chunk_cache_desc c;
+    int rc;
+    memset(&d, 0, sizeof d);
+    memset(&l, 0, sizeof l);
+    memset(&c, 0, sizeof c);
+    printf("sizeof gca_desc=%u lmk_desc=%u chunk_cache_desc=%u version=%d\n", (unsigned)sizeof d, (unsigned)sizeof l,
+           (unsigned)sizeof c, gca_version());
+    rc = gca_fwd(NULL, NULL, NULL, NULL, NULL, NULL, NULL, NULL);
+    printf("gca_fwd(NULL desc) -> %d (%s)\n", rc, gca_strerror(rc));
+    d.dtype = GCA_BF16; d.w_dtype = GCA_F32; d.Z = 4; d.Hq = 3; d.Hkv = 2; d.K = 2; d.Q_CTX = 64; d.K_CTX = 64; d.D = 64;
+    d.sm_scale = 0.125f;
+    rc = gca_fwd(&d, &d, &d, &d, &d, &d, NULL, NULL);          /* Hq % Hkv != 0 */
+    printf("gca_fwd(bad heads) -> %d (%s)\n", rc, gca_strerror(rc));
+    printf("bwd workspace for a bad descriptor: %lu\n", (unsigned long)gca_bwd_workspace_bytes(&d));
+    l.dtype = GCA_F32; l.topk = 8; l.N = 1; l.C = 4; l.E = 2; l.Dm = 8; l.causal = 1; l.hidden_size = 8.0f;
+    rc = lmk_score(&l, &l, &l, &l, NULL);                      /* causal with more rows than candidates */
+    printf("lmk_score(C > E) -> %d (%s)\n", rc, gca_strerror(rc));
+    c.dtype = GCA_F32; c.N = 1; c.capacity = 2; c.count = 1; c.n_new = 2; c.S = 8; c.Dm = 16;
+    rc = chunk_cache_append(&c, &c, &c, NULL, &c, &c, NULL, NULL);   /* 1 + 2 > capacity */
+    printf("chunk_cache_append(overflow) -> %d (%s)\n", rc, gca_strerror(rc));
+    return 0;
+}

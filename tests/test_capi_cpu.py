@@ -156,3 +156,28 @@ def test_manager_state_logic_on_cpu():
     import pytest
     with pytest.raises(AssertionError):
         m.append(torch.zeros(1, 1, 8, 16), torch.zeros(1, 1, 8, 16), torch.zeros(1, 1, 4))   # CPU tensors: no fallback
+
+
+def test_header_is_c99_and_links_from_plain_c(tmp_path):
+    """include/gca_hip.h compiles as strict C99, a C program links against the library and gets the same
+    struct sizes as the ctypes binding and the documented status codes (no GPU work is started)."""
+    import ctypes
+    import os
+    import shutil
+    import subprocess
+    from gca_hip import _lib
+    if shutil.which("gcc") is None:
+        import pytest
+        pytest.skip("no gcc")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    exe = str(tmp_path / "abi_check")
+    subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(root, "include"),
+                    os.path.join(root, "tests", "c", "abi_check.c"), "-o", exe, "-L", libdir, "-lgca_hip",
+                    "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib", "-Wl,--allow-shlib-undefined"], check=True)
+    out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout
+    assert f"sizeof gca_desc={ctypes.sizeof(_lib.GcaDesc)} lmk_desc={ctypes.sizeof(_lib.LmkDesc)} " \
+           f"chunk_cache_desc={ctypes.sizeof(_lib.ChunkCacheDesc)} version={_lib.lib().gca_version()}" in out
+    assert "gca_fwd(NULL desc) -> 1" in out and "gca_fwd(bad heads) -> 2" in out
+    assert "bwd workspace for a bad descriptor: 0" in out
+    assert "lmk_score(C > E) -> 2" in out and "chunk_cache_append(overflow) -> 2" in out
