@@ -202,8 +202,10 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
     constexpr int KS = D / 16, DB = D / 32;
     constexpr int RB = D * 2, TILE = 64 * RB, BUF = 2 * TILE;   // Q tile then dO tile
     __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * BUF];
-    __shared__ __attribute__((aligned(256))) float s_lse[2][64];
-    __shared__ __attribute__((aligned(256))) float s_dl[2][64];
+    // per wavefront and buffer: the unit's lse / delta rows, rewritten in place at the start of the unit into the
+    // exponent bias log2(w) - lse and -sm_scale * delta, so the element loop needs no per-element sub / mul for them
+    __shared__ __attribute__((aligned(256))) float s_lse[2][2][64];
+    __shared__ __attribute__((aligned(256))) float s_dl[2][2][64];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, kbw = tid >> 6;     // kbw: which 32 key rows this wavefront owns
@@ -304,8 +306,8 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
         unsigned char* nb = smem + buf * BUF;
         loader.issue(q + qoff, nb);
         loader.issue(dout + qoff, nb + TILE);
-        if (kbw == 0) async_row64(lse + loffq, s_lse[buf], lane);
-        else async_row64(delta + loffq, s_dl[buf], lane);
+        async_row64(lse + loffq, s_lse[kbw][buf], lane);
+        async_row64(delta + loffq, s_dl[kbw][buf], lane);
         return load_w(w, w_is_bf16, z * p.K + j);
     };
 
@@ -326,6 +328,10 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
         const float lw = __builtin_amdgcn_logf(w_cur);
 
         if (w_cur > 0.f) {
+        // this wavefront's copy of the rows: lse -> log2(w) - lse, delta -> -sm_scale * delta (LDS keeps a
+        // wavefront's own write and later reads in order, no barrier needed)
+        s_lse[kbw][buf][lane] = lw - s_lse[kbw][buf][lane];
+        s_dl[kbw][buf][lane] = -p.sm_scale * s_dl[kbw][buf][lane];
 #pragma unroll
         for (int qt = 0; qt < 2; ++qt) {
             // S = Q K^T, dP = dO V^T for 32 query rows: queries in registers, key n in the lane
@@ -343,14 +349,14 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
 #pragma unroll
             for (int a = 0; a < 4; ++a) {
                 // registers 4a .. 4a+3 are queries 32*qt + 8a + 4h + 0..3
-                f32x4 l4 = *reinterpret_cast<const f32x4*>(&s_lse[buf][32 * qt + 8 * a + 4 * h]);
-                f32x4 d4 = *reinterpret_cast<const f32x4*>(&s_dl[buf][32 * qt + 8 * a + 4 * h]);
+                f32x4 l4 = *reinterpret_cast<const f32x4*>(&s_lse[kbw][buf][32 * qt + 8 * a + 4 * h]);
+                f32x4 d4 = *reinterpret_cast<const f32x4*>(&s_dl[kbw][buf][32 * qt + 8 * a + 4 * h]);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int r = 4 * a + e;
-                    const float pw = __builtin_amdgcn_exp2f(fmaf(s[r], c, lw - l4[e]));
+                    const float pw = __builtin_amdgcn_exp2f(fmaf(s[r], c, l4[e]));
                     pA[r >> 3][r & 7] = (__bf16)pw;
-                    dsA[r >> 3][r & 7] = (__bf16)(pw * fmaf(dp[r], p.sm_scale, -d4[e] * p.sm_scale));
+                    dsA[r >> 3][r & 7] = (__bf16)(pw * fmaf(dp[r], p.sm_scale, d4[e]));
                 }
             }
             // dV += P~^T dO, dK += dS^T Q over these 32 queries (two 16-query reduction steps)
