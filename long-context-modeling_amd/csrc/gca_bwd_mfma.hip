@@ -100,10 +100,16 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
     const int fsw = swz(n);
     const int64_t lrow = (z * p.Hq + hq) * (int64_t)p.K * p.Q_CTX + q0 + n;
 
+    // The row's lse is requested one chunk ahead, so that it has arrived with the wait that ends the previous
+    // chunk: vector-memory operations retire in order, and a value requested and used inside a chunk would make
+    // the wavefront sit out the tile copies issued around it.
+    float lse_next = lse[lrow];
     for (int j = 0; j < p.K; ++j) {
         const int buf = j & 1;
         const bool more = j + 1 < p.K;
+        const float lse_cur = lse_next;
         if (more) {
+            lse_next = lse[lrow + (int64_t)(j + 1) * p.Q_CTX];
             // the other K buffer was last read in iteration j-1, which every wavefront has left
             int64_t rs;
             loader.issue(chunk_base_n(p, k, indices, nseq, z, hk, j + 1, rs), smem + (buf ^ 1) * TILE);
@@ -112,7 +118,7 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
         // A slot of weight 0 gives dS = 0: its P is left unscaled (delta is still needed) and the dQ product skipped.
         const float mult = load_w(w, w_is_bf16, z * p.K + j) * p.sm_scale;
         const bool live = mult > 0.f;
-        const float eoff = lse[lrow + (int64_t)j * p.Q_CTX] - (live ? __builtin_amdgcn_logf(mult) : 0.f);
+        const float eoff = lse_cur - (live ? __builtin_amdgcn_logf(mult) : 0.f);
         const float dscale = live ? 1.f / mult : 1.f;
         const unsigned char* kb = smem + buf * TILE;
         const unsigned char* vb = smem + 2 * TILE;
@@ -288,7 +294,7 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
         qrow0 = (u % nqt) * 64;
         hq = hk * p.G + g;
         if (INDEXED) {
-            const int ref = ws.refs[list0 + u / upr];
+            const int ref = load_uniform_int(ws.refs + list0 + u / upr);
             z = ref / p.K;
             j = ref % p.K;
         } else {
@@ -501,7 +507,7 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
         qrow0 = (u % nqt) * 64;
         hq = hk * p.G + g;
         if (INDEXED) {
-            const int ref = ws.refs[list0 + u / upr];
+            const int ref = load_uniform_int(ws.refs + list0 + u / upr);
             z = ref / p.K;
             j = ref % p.K;
         } else {

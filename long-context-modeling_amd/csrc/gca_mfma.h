@@ -63,6 +63,28 @@ struct TrLane {
     }
 };
 
+// One asynchronous global -> LDS copy instruction, written as assembly on purpose.  Through the compiler's builtin
+// the copy is known to write LDS, and because the tile buffers are slices of one LDS array the compiler then
+// puts "wait for every outstanding vector-memory operation" in front of the next LDS read it cannot tell apart
+// from the destination -- i.e. right after a prefetch is issued the wavefront would wait for it, and the copy
+// of the NEXT tile could never overlap the math on the current one.  Here the kernels order copies and reads
+// themselves (wait_async_tiles() + barrier before a buffer is read, barrier before it is refilled); waits the
+// compiler computes for its own loads stay valid, they can only become more conservative.
+// lds_addr must be wavefront-uniform: lane l's 16 (or 4) bytes land at lds_addr + 16*l (4*l).
+__device__ __forceinline__ unsigned lds_offset_of(const void* lds_ptr) {
+    return (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(uintptr_t)lds_ptr);   // low 32 bits = LDS offset
+}
+// (M0, which carries the LDS address, is written and consumed inside the block; the compiler keeps nothing in it
+// across other instructions of these kernels.)
+__device__ __forceinline__ void lds_dma_b128(const void* gptr, unsigned lds_addr) {
+    const int a = __builtin_amdgcn_readfirstlane((int)lds_addr);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(a), "v"(gptr) : "memory");
+}
+__device__ __forceinline__ void lds_dma_b32(const void* gptr, unsigned lds_addr) {
+    const int a = __builtin_amdgcn_readfirstlane((int)lds_addr);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(a), "v"(gptr) : "memory");
+}
+
 // Asynchronous global -> LDS copy of a ROWS x D bf16 tile (rows `rs` elements apart in global memory)
 // into a swizzled LDS tile, with global_load_lds_dwordx4: lane l of an instruction deposits its 16 bytes
 // at lds_base + 16*l, so one instruction fills 1 KB = 64*16/RB consecutive tile rows.  The swizzle is
@@ -90,19 +112,15 @@ struct TileLoader {
         }
     }
     __device__ __forceinline__ void issue(const uint16_t* tile, unsigned char* lds_tile) const {
-        typedef __attribute__((address_space(3))) void lds_void;
-        typedef __attribute__((address_space(1))) const void gbl_void;
+        const unsigned base = lds_offset_of(lds_tile) + wave * 1024;
 #pragma unroll
-        for (int i = 0; i < NI; ++i)
-            __builtin_amdgcn_global_load_lds((gbl_void*)(tile + goff[i]), (lds_void*)(lds_tile + (i * NW + wave) * 1024), 16, 0, 0);
+        for (int i = 0; i < NI; ++i) lds_dma_b128(tile + goff[i], base + i * NW * 1024);
     }
 };
 
 // 64 floats -> LDS (one wavefront, lane l writes element l)
 __device__ __forceinline__ void async_row64(const float* src, float* lds_dst, int lane) {
-    typedef __attribute__((address_space(3))) void lds_void;
-    typedef __attribute__((address_space(1))) const void gbl_void;
-    __builtin_amdgcn_global_load_lds((gbl_void*)(src + lane), (lds_void*)lds_dst, 4, 0, 0);
+    lds_dma_b32(src + lane, lds_offset_of(lds_dst));
 }
 
 // all outstanding global_load_lds of this wavefront have landed (vmcnt = 0; other counters untouched)
@@ -129,8 +147,24 @@ __device__ __forceinline__ int64_t xcd_logical(int64_t bid, int64_t total) {
 }
 inline int64_t xcd_grid(int64_t total) { return (total + NUM_XCD - 1) / NUM_XCD * NUM_XCD; }
 
+// Wavefront-uniform read of an int that no kernel of the same launch writes, through the scalar cache: the
+// compiler otherwise turns a uniform read through a plain pointer into a vector load plus "wait for every
+// outstanding vector-memory operation", which also waits for the tile copies in flight.
+__device__ __forceinline__ int load_uniform_int(const int* ptr) {
+    typedef __attribute__((address_space(4))) const int cint;
+    return *(cint*)ptr;
+}
+
+// Weight i of a (Z, K) array, i wavefront-uniform, read through the scalar cache (a 16-bit vector load here would
+// make the wavefront wait for every vector-memory operation in flight, tile copies included).
 __device__ __forceinline__ float load_w(const void* w, int w_is_bf16, int64_t i) {
-    return w_is_bf16 ? bf16_bits_to_f(((const uint16_t*)w)[i]) : ((const float*)w)[i];
+    typedef __attribute__((address_space(4))) const uint32_t cu32;
+    if (w_is_bf16) {
+        const uintptr_t addr = (uintptr_t)w + 2 * (uintptr_t)i;      // the aligned dword holding element i
+        const uint32_t word = *(cu32*)(addr & ~(uintptr_t)3);
+        return bf16_bits_to_f((addr & 2) ? (word >> 16) : (word & 0xffffu));
+    }
+    return __uint_as_float(((cu32*)w)[i]);
 }
 
 __device__ __forceinline__ uint16_t bf16_bits(float x) {
