@@ -210,16 +210,14 @@ lmk_score_mfma_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const uint16_
         b0off[i] = (nb * d.lmk_k_rows + min(e0 + row, d.E - 1)) * d.Dm + lp * 8;
         b1off[i] = (nb * d.lmk_k_rows + min(e0 + 64 + row, d.E - 1)) * d.Dm + lp * 8;
     }
-    typedef __attribute__((address_space(3))) void lds_void;
-    typedef __attribute__((address_space(1))) const void gbl_void;
     auto issue = [&](int k0, int buf) {
-        unsigned char* base = smem + buf * BUF;
+        const unsigned base = lds_offset_of(smem + buf * BUF) + wave * 1024;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            const int lo = (i * 4 + wave) * 1024;
-            __builtin_amdgcn_global_load_lds((gbl_void*)(lq + aoff[i] + k0), (lds_void*)(base + lo), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((gbl_void*)(lk + b0off[i] + k0), (lds_void*)(base + TILE + lo), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((gbl_void*)(lk + b1off[i] + k0), (lds_void*)(base + 2 * TILE + lo), 16, 0, 0);
+            const unsigned lo = base + i * 4 * 1024;
+            lds_dma_b128(lq + aoff[i] + k0, lo);
+            lds_dma_b128(lk + b0off[i] + k0, lo + TILE);
+            lds_dma_b128(lk + b1off[i] + k0, lo + 2 * TILE);
         }
     };
     f32x16 acc[2];
