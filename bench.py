@@ -28,7 +28,7 @@ for _p in (ROOT, os.path.join(ROOT, "long-context-modeling_amd")):
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the three main kernels at config 2, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled by the same counters' readings for a 1 GiB device copy (summary kept under profiles/)
-MEASURED_TRAFFIC_GB = {"gca_fwd_mfma_kernel": 1.150, "gca_bwd_dq_mfma_kernel": 1.632, "gca_bwd_dkdv2_mfma_kernel": 1.843}
+MEASURED_TRAFFIC_GB = {"gca_fwd_mfma_kernel": 1.138, "gca_bwd_dq_mfma_kernel": 1.551, "gca_bwd_dkdv2_mfma_kernel": 1.776}
 
 
 def log(*a):
