@@ -68,3 +68,34 @@ def test_rows_with_no_weight_and_unretrieved_chunks():
     o, dq, dk, dv, dw = _case(N, C, 4, 4, 64, 64, K, torch.bfloat16, seed=330, idx=idx, w=w)
     assert o[::2].abs().max() == 0 and dq[::2].abs().max() == 0
     assert dk[:, 2:].abs().max() == 0 and dv[:, 2:].abs().max() == 0
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_seeded_random_shapes_gathered_form(seed):
+    """Shapes drawn from a seeded generator (head counts, group sizes, slot counts, ragged query / key row counts,
+    every head dim, both dtypes, both kernel families where the shape allows) against the float64 oracle."""
+    import gca_hip
+    from gca_hip import gca as G
+    from helpers import gca_inputs, oracle64
+    g = torch.Generator().manual_seed(1000 + seed)
+    pick = lambda xs: xs[int(torch.randint(0, len(xs), (1,), generator=g))]
+    d = pick([16, 32, 64, 64, 128, 256])
+    Hkv = pick([1, 2, 3])
+    Hq = Hkv * pick([1, 2, 4])
+    K = pick([1, 2, 3, 5, 8])
+    mfma_like = pick([True, False])
+    Q = 64 * pick([1, 2]) if mfma_like else pick([1, 2, 7, 33, 64, 100])
+    S = 64 if mfma_like else pick([16, 48, 64, 80])
+    Z = pick([1, 2, 5])
+    dtype = pick([torch.float32, torch.bfloat16])
+    sm_n = pick([0.0, 1.0])
+    q, k, v, w, do = gca_inputs(Z, Hq, Hkv, K, Q, S, d, dtype, seed=2000 + seed)
+    ref = oracle64(q, k, v, w, do, d ** -0.5, sm_n)
+    qd, kd, vd, wd = [t.cuda().requires_grad_() for t in (q, k, v, w)]
+    o = gca_hip.attention(qd, kd, vd, wd, d ** -0.5, sm_n)
+    o.backward(do.cuda())
+    tol = TOL[dtype]
+    for name, a, r in zip("o dq dk dv dw".split(), (o, qd.grad, kd.grad, vd.grad, wd.grad), ref):
+        assert torch.isfinite(a.float()).all(), (name, Z, Hq, Hkv, K, Q, S, d, dtype)
+        lim = tol if (name != "dw" or dtype == torch.float32) else 3e-2
+        assert rel_err(a, r) <= lim, (name, Z, Hq, Hkv, K, Q, S, d, dtype, sm_n)
