@@ -28,16 +28,13 @@
 //    partial tiles; a small reduce launch adds those up in segment order.
 //
 // dw[z, j] = sum over heads and rows of delta (shared launch_dw).
-#include <cstdlib>
 #include "gca_mfma.h"
 #include "gca_lists.h"
 
 namespace gca {
 
-
-static int seg_max_from_env() { const char* e = getenv("GCA_SEG_MAX"); const int v = e ? atoi(e) : 0; return v > 0 ? v : 32; }
-// references per dkdv workgroup in the indexed form (GCA_SEG_MAX overrides, for tuning)
-static const int SEG_MAX = seg_max_from_env();
+// references per dkdv workgroup in the indexed form: longer lists are cut into segments of this many
+constexpr int SEG_MAX = 32;
 
 // ------------------------------------------------------------------------------------------- dq
 
@@ -114,12 +111,14 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
             int64_t rs;
             loader.issue(chunk_base_n(p, k, indices, nseq, z, hk, j + 1, rs), smem + (buf ^ 1) * TILE);
         }
-        // mult = w_j * sm_scale multiplies dS; it rides in the exponent: Pm = mult * P = exp2(c S - lse + log2 mult).
-        // A slot of weight 0 gives dS = 0: its P is left unscaled (delta is still needed) and the dQ product skipped.
+        // mult = w_j * sm_scale multiplies dS; its magnitude rides in the exponent: Pm = |mult| P = exp2(c S - lse + log2 |mult|),
+        // its sign is put on the rounded dS operand.  A slot of weight 0 gives dS = 0: its P is left unscaled (delta is
+        // still needed) and the dQ product skipped.
         const float mult = load_w(w, w_is_bf16, z * p.K + j) * p.sm_scale;
-        const bool live = mult > 0.f;
-        const float eoff = lse_cur - (live ? __builtin_amdgcn_logf(mult) : 0.f);
-        const float dscale = live ? 1.f / mult : 1.f;
+        const float amult = fabsf(mult);
+        const bool live = amult > 0.f;
+        const float eoff = lse_cur - (live ? __builtin_amdgcn_logf(amult) : 0.f);
+        const float dscale = live ? 1.f / amult : 1.f;
         const unsigned char* kb = smem + buf * TILE;
         const unsigned char* vb = smem + 2 * TILE;
 
@@ -164,6 +163,10 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
                     const int r = 8 * (t4 & 1) + s;
                     dsA[t4][s] = (__bf16)(st[t4 >> 1][r] * (dpt[t4 >> 1][r] - dsum));
                 }
+            if (mult < 0.f) {
+#pragma unroll
+                for (int t4 = 0; t4 < 4; ++t4) dsA[t4] = negate_bf16x8(dsA[t4]);
+            }
 #pragma unroll
             for (int t4 = 0; t4 < 4; ++t4)
 #pragma unroll
@@ -330,10 +333,12 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
         if (more) w_next = issue_unit(u + 1, buf ^ 1);   // that buffer was last read in iteration u-1
         const unsigned char* qbuf = smem + buf * BUF;
         const unsigned char* dobuf = qbuf + TILE;
-        // P~ = w P rides in the exponent (exp2(c S - lse + log2 w)); a slot of weight 0 adds nothing to dk, dv
-        const float lw = __builtin_amdgcn_logf(w_cur);
+        // |w| rides in the exponent (P~ = exp2(c S - lse + log2 |w|)), the sign of w goes on the rounded operands;
+        // a slot of weight 0 adds nothing to dk, dv
+        const float lw = __builtin_amdgcn_logf(fabsf(w_cur));
+        const bool wneg = w_cur < 0.f;
 
-        if (w_cur > 0.f) {
+        if (w_cur != 0.f) {
         // this wavefront's copy of the rows: lse -> log2(w) - lse, delta -> -sm_scale * delta (LDS keeps a
         // wavefront's own write and later reads in order, no barrier needed)
         s_lse[kbw][buf][lane] = lw - s_lse[kbw][buf][lane];
@@ -364,6 +369,10 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
                     pA[r >> 3][r & 7] = (__bf16)pw;
                     dsA[r >> 3][r & 7] = (__bf16)(pw * fmaf(dp[r], p.sm_scale, d4[e]));
                 }
+            }
+            if (wneg) {
+#pragma unroll
+                for (int t2 = 0; t2 < 2; ++t2) { pA[t2] = negate_bf16x8(pA[t2]); dsA[t2] = negate_bf16x8(dsA[t2]); }
             }
             // dV += P~^T dO, dK += dS^T Q over these 32 queries (two 16-query reduction steps)
 #pragma unroll
@@ -556,9 +565,10 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
         if (more) w_next = issue_unit(u + 1, buf ^ 1);   // that buffer was last read in iteration u-1
         const unsigned char* qbuf = smem + buf * BUF;
         const unsigned char* dobuf = qbuf + TILE;
-        const bool live = w_cur > 0.f;      // a slot of weight 0 adds nothing to dk, dv
-        // P~ = w P rides in the exponent: exp2(c S - lse + log2 w)
-        const float lw = __builtin_amdgcn_logf(w_cur);
+        const bool live = w_cur != 0.f;     // a slot of weight 0 adds nothing to dk, dv
+        // |w| rides in the exponent (P~ = exp2(c S - lse + log2 |w|)), the sign of w goes on the rounded operands
+        const float lw = __builtin_amdgcn_logf(fabsf(w_cur));
+        const bool wneg = w_cur < 0.f;
 
         if (live) {
             // ---- phase 1: S = Q K^T, dP = dO V^T for query rows 32*sub .. +31 against key rows 32*kbw .. +31
@@ -582,6 +592,10 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
                     pA[r >> 3][r & 7] = (__bf16)pw;
                     dsA[r >> 3][r & 7] = (__bf16)(pw * fmaf(dp[r], p.sm_scale, -d_cur[a][e] * p.sm_scale));
                 }
+            if (wneg) {
+#pragma unroll
+                for (int t2 = 0; t2 < 2; ++t2) { pA[t2] = negate_bf16x8(pA[t2]); dsA[t2] = negate_bf16x8(dsA[t2]); }
+            }
             // hand the A operands of 16-query steps 2*sub, 2*sub+1 to the phase-2 owners, lane for lane
 #pragma unroll
             for (int t2 = 0; t2 < 2; ++t2) {

@@ -74,16 +74,20 @@ struct TrLane {
 __device__ __forceinline__ unsigned lds_offset_of(const void* lds_ptr) {
     return (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(uintptr_t)lds_ptr);   // low 32 bits = LDS offset
 }
-// (M0, which carries the LDS address, is written and consumed inside the block; the compiler keeps nothing in it
-// across other instructions of these kernels.)
+// M0 carries the LDS address; it is written and consumed inside the block and named as clobbered, so the
+// compiler's own M0 initialisations are never merged across one of these blocks.  (clang notes that M0 is a
+// reserved register it will not save around the statement -- which is what is wanted here.)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void lds_dma_b128(const void* gptr, unsigned lds_addr) {
     const int a = __builtin_amdgcn_readfirstlane((int)lds_addr);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(a), "v"(gptr) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(a), "v"(gptr) : "memory", "m0");
 }
 __device__ __forceinline__ void lds_dma_b32(const void* gptr, unsigned lds_addr) {
     const int a = __builtin_amdgcn_readfirstlane((int)lds_addr);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(a), "v"(gptr) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(a), "v"(gptr) : "memory", "m0");
 }
+#pragma clang diagnostic pop
 
 // Asynchronous global -> LDS copy of a ROWS x D bf16 tile (rows `rs` elements apart in global memory)
 // into a swizzled LDS tile, with global_load_lds_dwordx4: lane l of an instruction deposits its 16 bytes
@@ -165,6 +169,14 @@ __device__ __forceinline__ float load_w(const void* w, int w_is_bf16, int64_t i)
         return bf16_bits_to_f((addr & 2) ? (word >> 16) : (word & 0xffffu));
     }
     return __uint_as_float(((cu32*)w)[i]);
+}
+
+// flips the sign of all eight bf16 values (four 32-bit XORs)
+__device__ __forceinline__ bf16x8 negate_bf16x8(bf16x8 v) {
+    union { bf16x8 b; u32x4 u; } x;
+    x.b = v;
+    x.u ^= 0x80008000u;
+    return x.b;
 }
 
 __device__ __forceinline__ uint16_t bf16_bits(float x) {

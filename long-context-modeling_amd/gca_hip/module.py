@@ -6,6 +6,16 @@ attention runs on the projection's own (N, C, S, Hq*d) layout: the reference's t
 copies around the kernel (DRT.py:366-378, :384) and the zero-filled output copy (DRT.py:387-394) are gone,
 and because the kernels read retrieved chunks from the cache by index, the one retrieval of a layer group
 (DRT.py:816-822) serves all its layers with no gathered copy at all.
+
+Softmax-off-by-one.  The reference module hands ``sm_n = 1.0`` to its kernels when ``enable_softmax_one`` is
+set (DRT.py:317-318, :380-382), but inside those kernels the value has no numerical effect: the running
+denominator starts at ``sm_n`` and is multiplied by ``exp2(-inf) = 0`` on the first key tile
+(ltriton/gca.py:186-187 with :48-49).  The model's "+1" is the zeroed landmark row of every cached chunk
+(DRT.py:771-779: a key of logit 0 with value 0).  ``sm_n_mode = "reference"`` (default) therefore runs the
+kernels with ``sm_n = 0`` and expects the cache to hold the zeroed row (``ChunkKVManager.append(...,
+landmark_row="zero")``), which reproduces the reference on its own checkpoints.  ``"functional"`` passes
+``sm_n`` on to the kernels (denominator ``sm_n + sum exp``) for caches stored with ``landmark_row="drop"``;
+using it on a cache that also holds the zeroed row would count the "+1" twice.
 """
 from __future__ import annotations
 
@@ -17,7 +27,7 @@ from .gca import attention_tokens
 
 class GroupCrossAttention(nn.Module):
     def __init__(self, hidden_size, num_heads, enc_chunk_size=64, chunk_topk=8, rms_norm_eps=1e-6,
-                 attention_bias=False, enable_softmax_one=False):
+                 attention_bias=False, enable_softmax_one=False, sm_n_mode="reference"):
         super().__init__()
         self.hidden_size = hidden_size
         self.num_heads = num_heads
@@ -27,7 +37,14 @@ class GroupCrossAttention(nn.Module):
         self.pre_norm = nn.RMSNorm(hidden_size, eps=rms_norm_eps)
         self.q_proj = nn.Linear(hidden_size, num_heads * self.head_dim, bias=attention_bias)
         self.o_proj = nn.Linear(hidden_size, num_heads * self.head_dim, bias=attention_bias)
-        self.sm_n = 1.0 if enable_softmax_one else 0.0            # DRT.py:318-319
+        self.sm_n = 1.0 if enable_softmax_one else 0.0            # DRT.py:317-318
+        assert sm_n_mode in ("reference", "functional"), sm_n_mode
+        self.sm_n_mode = sm_n_mode
+
+    @property
+    def kernel_sm_n(self):
+        """What the kernels get: 0 in "reference" mode (the argument is inert in the reference's kernels)."""
+        return self.sm_n if self.sm_n_mode == "functional" else 0.0
 
     def forward(self, hidden_states, chunk_kvs, indices, weights):
         """hidden_states (N, C, S, dim); ``chunk_kvs`` a ChunkKVManager (or a (k_store, v_store) pair);
@@ -38,7 +55,7 @@ class GroupCrossAttention(nn.Module):
             return torch.zeros((N, C * S, dim), device=hidden_states.device, dtype=hidden_states.dtype)
         k_store, v_store = (chunk_kvs.k_store, chunk_kvs.v_store) if hasattr(chunk_kvs, "k_store") else chunk_kvs
         q = self.q_proj(self.pre_norm(hidden_states))             # (N, C, S, Hq*d), read in place by the kernel
-        vals = attention_tokens(q.contiguous(), k_store, v_store, indices, weights, self.num_heads, self.sm_n)
+        vals = attention_tokens(q.contiguous(), k_store, v_store, indices, weights, self.num_heads, self.kernel_sm_n)
         o = self.o_proj(vals)                                     # chunk 0 of vals is zero
         if self.o_proj.bias is not None:
             keep = torch.ones((1, C, 1, 1), device=o.device, dtype=o.dtype)
@@ -52,5 +69,5 @@ class GroupCrossAttention(nn.Module):
         (DRT.py:345-398 with chunk_size == 1, :825-831).  Returns (N, Q, dim)."""
         N, Q, dim = hidden_states.shape
         q = self.q_proj(self.pre_norm(hidden_states)).view(N, Q, self.num_heads, self.head_dim)
-        vals = chunk_kvs.decode_attention(q.transpose(1, 2).contiguous(), group_idx, self.sm_n)   # (N, Hq, Q, d)
+        vals = chunk_kvs.decode_attention(q.transpose(1, 2).contiguous(), group_idx, self.kernel_sm_n)   # (N, Hq, Q, d)
         return self.o_proj(vals.transpose(1, 2).reshape(N, Q, self.num_heads * self.head_dim))

@@ -263,11 +263,18 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
 
 
 def gca_module_forward(hidden, chunk_k, chunk_v, indices, weights, norm_w, eps, wq, bq, wo, bo, num_heads: int,
-                       num_kv_heads: int, sm_n: float = 0.0):
+                       num_kv_heads: int, sm_n: float = 0.0, sm_n_functional: bool = False):
     """TritonGroupCrossAttention.forward for chunk_size > 1, step by step (model/DRT.py:345-398):
     pre_norm -> q_proj -> 'N D S (h d) -> N D h S d' -> drop chunk 0 -> '(N D) h S d' -> kernel with
     sm_scale = 1/sqrt(d) -> '(N D) h S d -> N (D S) (h d)' -> o_proj -> zero-filled result whose last
-    (C-1)*S rows are the output.  hidden (N, C, S, dim); indices/weights (N, C, kk) from the retrieval."""
+    (C-1)*S rows are the output.  hidden (N, C, S, dim); indices/weights (N, C, kk) from the retrieval.
+
+    ``sm_n`` is what the module passes to its kernel (1.0 with enable_softmax_one, model/DRT.py:317-318).  Inside
+    the reference's kernels it is numerically inert: the denominator starts at sm_n and is multiplied by
+    exp2(m_i - m_ij) = exp2(-inf) = 0 on the first key tile (ltriton/gca.py:186-187, :48-49); the model's "+1"
+    is the zeroed landmark row the caller stores in chunk_k / chunk_v (model/DRT.py:771-779).  So the
+    restatement evaluates the plain softmax whatever sm_n is; ``sm_n_functional=True`` states the other
+    reading (denominator sm_n + sum exp) for caches stored without that row."""
     N, C, S, dim = hidden.shape
     d = dim // num_heads
     x = rms_norm(hidden, norm_w, eps)
@@ -275,7 +282,7 @@ def gca_module_forward(hidden, chunk_k, chunk_v, indices, weights, norm_w, eps, 
     q = q.reshape(N, C, S, num_heads, d).permute(0, 1, 3, 2, 4)         # N D h S d
     q = q[:, 1:].reshape(N * (C - 1), num_heads, S, d)                  # model/DRT.py:369-372
     k, v, w = gather_chunks(chunk_k, chunk_v, indices, weights, num_kv_heads)
-    vals = gca_forward(q, k, v, w, 1.0 / math.sqrt(d), sm_n)            # ((N D), h, S, d)
+    vals = gca_forward(q, k, v, w, 1.0 / math.sqrt(d), sm_n if sm_n_functional else 0.0)   # ((N D), h, S, d)
     vals = vals.reshape(N, C - 1, num_heads, S, d).permute(0, 1, 3, 2, 4).reshape(N, (C - 1) * S, num_heads * d)
     o = F.linear(vals, wo, bo)
     ret = torch.zeros((N, C * S, dim), dtype=o.dtype)

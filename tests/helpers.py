@@ -34,3 +34,59 @@ def oracle64(q, k, v, w, do, sm_scale, sm_n):
     o = orc.gca_forward(q, k, v, w, sm_scale, sm_n)
     dq, dk, dv, dw = orc.gca_backward(q, k, v, w, do, sm_scale, sm_n)
     return o, dq, dk, dv, dw
+
+
+def sampled_oracle_check(q, ck, cv, idx, w, do, got, Hkv, sm_scale, sm_n, z_rows, chunks=(), tol=2e-2, q_of=None):
+    """Oracle comparison of a full-size indexed run on a sample of it, on the host in float64.
+
+    q, do (Z, Hq, S, d), ck, cv (N, C, S, Hkv*d), idx, w (Z, K) live on the GPU; ``got`` = (o, dq, dk_cache,
+    dv_cache, dw) from the kernels (dq .. dw may be None for a forward-only run).  For every sampled query chunk z
+    (all its heads) the K retrieved chunks are gathered to the host and o, dq, dw compared; for every sampled
+    cache chunk (n, c) the contributions of all query chunks that retrieved it are summed by the oracle and
+    compared with that chunk's tile of dk_cache / dv_cache.  Error measure: max |err| / max |ref| per sampled
+    block."""
+    o, dq, dkc, dvc, dw = got
+    N, C, S, Dm = ck.shape
+    Z, Hq, _, d = q.shape
+    zpn = Z // N
+    K = idx.shape[1]
+
+    def gather(z):
+        n = z // zpn
+        ids = idx[z].clamp(0, C - 1)
+        k = ck[n, ids].reshape(K, S, Hkv, d).permute(2, 0, 1, 3)          # (Hkv, K, S, d)
+        v = cv[n, ids].reshape(K, S, Hkv, d).permute(2, 0, 1, 3)
+        return k.double().cpu(), v.double().cpu()
+
+    worst = {}
+
+    def note(name, a, r):
+        e = rel_err(a, r)
+        worst[name] = max(worst.get(name, 0.0), e)
+        assert e <= tol, f"{name}: rel err {e:.3e} > {tol}"
+
+    for z in z_rows:
+        k, v = gather(z)
+        qz, doz, wz = q[z:z + 1].double().cpu(), do[z:z + 1].double().cpu(), w[z:z + 1].double().cpu()
+        ref_o = orc.gca_forward(qz, k[None], v[None], wz, sm_scale, sm_n)
+        note("o", o[z:z + 1], ref_o)
+        if dq is not None:
+            rdq, _, _, rdw = orc.gca_backward(qz, k[None], v[None], wz, doz, sm_scale, sm_n)
+            note("dq", dq[z:z + 1], rdq)
+            note("dw", dw[z:z + 1], rdw)
+    for (n, c) in chunks:
+        rows = idx[n * zpn:(n + 1) * zpn].clamp(0, C - 1)
+        zz, jj = torch.nonzero(rows == c, as_tuple=True)
+        kt = ck[n, c].reshape(S, Hkv, d).permute(1, 0, 2).double().cpu()[None, :, None]      # (1, Hkv, 1, S, d)
+        vt = cv[n, c].reshape(S, Hkv, d).permute(1, 0, 2).double().cpu()[None, :, None]
+        rk, rv = torch.zeros_like(kt[0, :, 0]), torch.zeros_like(vt[0, :, 0])
+        for zi, j in zip(zz.tolist(), jj.tolist()):
+            z = n * zpn + zi
+            qz, doz = q[z:z + 1].double().cpu(), do[z:z + 1].double().cpu()
+            wz = w[z:z + 1, j:j + 1].double().cpu()
+            _, dk1, dv1, _ = orc.gca_backward(qz, kt, vt, wz, doz, sm_scale, sm_n)   # one slot: D_j needs only chunk j
+            rk += dk1[0, :, 0]
+            rv += dv1[0, :, 0]
+        note("dk_cache", dkc[n, c].reshape(S, Hkv, d).permute(1, 0, 2), rk)
+        note("dv_cache", dvc[n, c].reshape(S, Hkv, d).permute(1, 0, 2), rv)
+    return worst

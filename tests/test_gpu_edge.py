@@ -39,7 +39,7 @@ def _case(N, C, Hq, Hkv, S, d, K, dtype, seed, idx=None, w=None):
     for name, a, r in (("o", o, o_ref), ("dq", qd.grad, q64.grad), ("dk", ckd.grad, ck64.grad),
                        ("dv", cvd.grad, cv64.grad), ("dw", wd.grad, w64.grad)):
         assert torch.isfinite(a.float()).all(), name
-        assert rel_err(a, r) <= (tol if name != "dw" or dtype == torch.float32 else 3e-2), name
+        assert rel_err(a, r) <= tol, name
     return o, qd.grad, ckd.grad, cvd.grad, wd.grad
 
 
@@ -97,5 +97,42 @@ def test_seeded_random_shapes_gathered_form(seed):
     tol = TOL[dtype]
     for name, a, r in zip("o dq dk dv dw".split(), (o, qd.grad, kd.grad, vd.grad, wd.grad), ref):
         assert torch.isfinite(a.float()).all(), (name, Z, Hq, Hkv, K, Q, S, d, dtype)
-        lim = tol if (name != "dw" or dtype == torch.float32) else 3e-2
-        assert rel_err(a, r) <= lim, (name, Z, Hq, Hkv, K, Q, S, d, dtype, sm_n)
+        assert rel_err(a, r) <= tol, (name, Z, Hq, Hkv, K, Q, S, d, dtype, sm_n)
+
+
+@pytest.mark.parametrize("d,Hq,Hkv", [(64, 4, 2), (128, 4, 1), (64, 3, 3)])
+@pytest.mark.parametrize("path", ["mfma", "generic"])
+def test_mixed_sign_weights(d, Hq, Hkv, path):
+    """The fusion weights are a plain input of the drop-in (ltriton/gca.py:387, :474 multiply by them whatever their
+    sign): negative, zero and positive weights in one row, both kernel families, gathered and indexed form."""
+    import gca_hip
+    from gca_hip import gca as G
+    from helpers import gca_inputs, oracle64
+    Z, K, S = 5, 6, 64
+    q, k, v, w, do = gca_inputs(Z, Hq, Hkv, K, S, S, d, torch.bfloat16, seed=400 + d, w_dtype=torch.float32)
+    g = torch.Generator().manual_seed(401)
+    w = torch.randn(Z, K, generator=g)
+    w[:, 2] = 0.0
+    w[0] = -w[0].abs()                                   # a row of negative weights only
+    ref = oracle64(q, k, v, w, do, d ** -0.5, 1.0)
+    old = G.kernel_path
+    G.kernel_path = path
+    try:
+        qd, kd, vd, wd = [t.cuda().requires_grad_() for t in (q, k, v, w)]
+        o = gca_hip.attention(qd, kd, vd, wd, d ** -0.5, 1.0)
+        o.backward(do.cuda())
+        for name, a, r in zip("o dq dk dv dw".split(), (o, qd.grad, kd.grad, vd.grad, wd.grad), ref):
+            assert rel_err(a, r) <= 2e-2, (name, rel_err(a, r))
+        # indexed form: every (z, kv head, j) tile becomes a cache chunk of its own, so dk_cache must equal dk
+        kc = k.permute(0, 2, 3, 1, 4).reshape(1, Z * K, S, Hkv * d).contiguous()
+        vc = v.permute(0, 2, 3, 1, 4).reshape(1, Z * K, S, Hkv * d).contiguous()
+        idx = torch.arange(Z * K).view(Z, K)
+        qd, kd, vd, wd = [t.cuda().requires_grad_() for t in (q, kc, vc, w)]
+        o = gca_hip.attention_indexed(qd, kd, vd, idx.cuda(), wd, d ** -0.5, 1.0)
+        o.backward(do.cuda())
+        dk_i = kd.grad.view(Z, K, S, Hkv, d).permute(0, 3, 1, 2, 4)
+        dv_i = vd.grad.view(Z, K, S, Hkv, d).permute(0, 3, 1, 2, 4)
+        for name, a, r in zip("o dq dk dv dw".split(), (o, qd.grad, dk_i, dv_i, wd.grad), ref):
+            assert rel_err(a, r) <= 2e-2, ("indexed", name, rel_err(a, r))
+    finally:
+        G.kernel_path = old

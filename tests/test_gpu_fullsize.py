@@ -1,8 +1,10 @@
-"""Full-size checks at BASELINE.json's shapes, through properties that do not need the CPU oracle:
-agreement of the MFMA kernels with the independent generic (fp32-arithmetic) kernels, linearity in V,
-invariance under a permutation of the retrieval slots, the dw / delta identity, indexed == gathered,
-the needle of config 3, and scoring / top-k against torch's own device ops.  Tolerance for bf16
-comparisons: max |a-b| / max |b| <= 2e-2."""
+"""Full-size checks at BASELINE.json's shapes.  Two kinds: (1) the CPU oracle in float64 on a SAMPLE of the
+full-size run (whole query chunks with all their heads for o / dq / dw, whole cache chunks with every
+reference to them for dk / dv), and (2) properties that need no oracle: agreement of the MFMA kernels with the
+independent generic (fp32-arithmetic) kernels, linearity in V, invariance under a permutation of the retrieval
+slots, the dw / delta identity, indexed == gathered, the needle of config 3, scoring / top-k against torch's
+own device ops, and -- for the 16.7M-token cache of config 5a -- bit equality with the same call on a small
+cache holding copies of the selected chunks.  Tolerance for bf16 comparisons: max |a-b| / max |b| <= 2e-2."""
 import math
 
 import pytest
@@ -76,6 +78,118 @@ def test_cfg2_mfma_vs_generic_and_invariants():
     o_a = gca_hip.gca_kv_cache_indexed(q, ck, cv2, idx, w, 0.125, 1.0)
     o_s = gca_hip.gca_kv_cache_indexed(q, ck, (cv.float() + cv2.float()).bfloat16(), idx, w, 0.125, 1.0)
     assert _rel(o_s, o.float() + o_a.float()) <= 2e-2
+
+
+def _sample_rows(Z, zpn, n_rows, seed):
+    g = torch.Generator().manual_seed(seed)
+    rows = torch.randint(0, Z, (n_rows,), generator=g).tolist()
+    return sorted(set(rows + [0, zpn - 1, Z - 1]))           # first row (one visible chunk), a sequence's last, the very last
+
+
+@pytest.mark.parametrize("sm_n", [1.0, 0.0])
+def test_cfg2_full_size_sampled_oracle(sm_n):
+    """BASELINE config 2 at full size (B=8, 256 chunks, H=12, d=64, top-k 8, bf16) through retrieval + indexed
+    forward + backward; a sample of query chunks and cache chunks is recomputed by the float64 oracle."""
+    import gca_hip
+    from helpers import sampled_oracle_check
+    q, ck, cv, lq, lk, do = _cfg2(seed=11)
+    N, C, S, Dm = ck.shape
+    Z, H, _, d = q.shape
+    K = 8
+    _, indices, weights = gca_hip.landmark_retrieve(lq, lk, K, Dm)
+    idx = indices[:, :-1].reshape(Z, K).contiguous()
+    w = weights[:, :-1].reshape(Z, K).contiguous()
+    got = _run_indexed(q, ck, cv, idx, w, do, "mfma", sm_n=sm_n)
+    # cache chunks: an early one (retrieved by many later rows), a middle one, the last retrievable one, an unretrievable one
+    chunks = [(0, 0), (3, 100), (7, C - 2), (5, C - 1)]
+    worst = sampled_oracle_check(q, ck, cv, idx, w, do, got, H, 0.125, sm_n, _sample_rows(Z, C - 1, 5, 1), chunks)
+    print("cfg2 sampled oracle, worst rel err:", {k_: f"{v:.2e}" for k_, v in worst.items()})
+
+
+def test_cfg4_full_size_sampled_oracle():
+    """BASELINE config 4 at full size (B=4, 512 chunks, 32 query heads over 8 kv heads, d=128, top-k 16, bf16,
+    retrieval logits ~ N(0,1) given directly), fwd + bwd, sampled against the float64 oracle."""
+    import gca_hip
+    from helpers import sampled_oracle_check
+    N, C, Hq, Hkv, S, d, K = 4, 512, 32, 8, 64, 128, 16
+    g = torch.Generator(device=DEV).manual_seed(13)
+    Z = N * (C - 1)
+    q = (torch.randn(Z, Hq, S, d, device=DEV, generator=g) * 0.35).bfloat16()
+    ck = (torch.randn(N, C, S, Hkv * d, device=DEV, generator=g) * 0.35).bfloat16()
+    cv = (torch.randn(N, C, S, Hkv * d, device=DEV, generator=g) * 0.35).bfloat16()
+    do = torch.randn(Z, Hq, S, d, device=DEV, generator=g).bfloat16()
+    scores = torch.randn(N, C, C, device=DEV, generator=g).bfloat16()
+    indices, weights = gca_hip.landmark_topk(scores, K)
+    idx = indices[:, :-1].reshape(Z, K).contiguous()
+    w = weights[:, :-1].reshape(Z, K).contiguous()
+    a = [t.detach().clone().requires_grad_(True) for t in (q, ck, cv, w)]
+    o = gca_hip.attention_indexed(a[0], a[1], a[2], idx, a[3], d ** -0.5, 0.0)
+    got = (o.detach(),) + tuple(torch.autograd.grad(o, a, do))
+    worst = sampled_oracle_check(q, ck, cv, idx, w, do, got, Hkv, d ** -0.5, 0.0, _sample_rows(Z, C - 1, 3, 2),
+                                 [(0, 1), (2, 300), (3, C - 2)])
+    print("cfg4 sampled oracle, worst rel err:", {k_: f"{v:.2e}" for k_, v in worst.items()})
+
+
+def test_cfg3_full_size_forward_sampled_oracle():
+    """BASELINE config 3 at full size (B=1, 16384 chunks = 1M tokens, H=12, d=64, top-k 8, bf16): scoring + top-k +
+    forward over all 16383 query chunks; sampled rows against the float64 oracle, and the needle must be retrieved."""
+    import gca_hip
+    from helpers import sampled_oracle_check
+    N, C, H, S, d, K = 1, 16384, 12, 64, 64, 8
+    g = torch.Generator(device=DEV).manual_seed(17)
+    Z = C - 1
+    q = (torch.randn(Z, H, S, d, device=DEV, generator=g) * 0.5).bfloat16()
+    ck = (torch.randn(N, C, S, H * d, device=DEV, generator=g) * 0.5).bfloat16()
+    cv = (torch.randn(N, C, S, H * d, device=DEV, generator=g) * 0.5).bfloat16()
+    lk = (ck.float().mean(2) + 0.1 * torch.randn(N, C, H * d, device=DEV, generator=g)).bfloat16()
+    needle = 4321
+    direction = lk[0, needle].float()
+    lk[0, needle] = (4 * direction).bfloat16()
+    lq = (torch.randn(N, C, H * d, device=DEV, generator=g) + 0.5 * direction).bfloat16()
+    _, indices, weights = gca_hip.landmark_retrieve(lq, lk, K, H * d)
+    assert (indices[0, needle + 1:] == needle).any(-1).all()
+    idx = indices[:, :-1].reshape(Z, K).contiguous()
+    w = weights[:, :-1].reshape(Z, K).contiguous()
+    o = gca_hip.gca_kv_cache_indexed(q, ck, cv, idx, w, 0.125, 1.0)
+    assert torch.isfinite(o.float()).all()
+    worst = sampled_oracle_check(q, ck, cv, idx, w, q, (o, None, None, None, None), H, 0.125, 1.0,
+                                 _sample_rows(Z, Z, 6, 3))
+    print("cfg3 sampled oracle, worst rel err:", {k_: f"{v:.2e}" for k_, v in worst.items()})
+
+
+def test_cfg5a_attention_over_16M_token_cache():
+    """BASELINE config 5a: B=1 with 262144 cached chunks (16.7M tokens).  Each cache is 1.29e10 elements (25.8 GB), so
+    chunks with id > 43690 start beyond element 2^32: the indexed forward must address them with 64-bit offsets.
+    Checked bit for bit against the same call on an 8-chunk cache holding copies of the selected chunks, and against
+    the float64 oracle on those chunks."""
+    import gca_hip
+    from helpers import rel_err
+    from oracle import gca_oracle as orc
+    N, E, H, S, d, K = 1, 262144, 12, 64, 64, 8
+    ck = torch.empty((N, E, S, H * d), device=DEV, dtype=torch.bfloat16)
+    cv = torch.empty((N, E, S, H * d), device=DEV, dtype=torch.bfloat16)
+    g = torch.Generator(device=DEV).manual_seed(19)
+    slab = 8192
+    for a in range(0, E, slab):                     # filled in place, slab by slab: no float32 copy of 12.9e9 elements
+        ck[:, a:a + slab].normal_(0, 0.5, generator=g)
+        cv[:, a:a + slab].normal_(0, 0.5, generator=g)
+    ids = torch.tensor([[5, 43691, 100000, 131072, 200000, E - 1, 43690, 65536]], device=DEV)
+    assert int(ids.max()) * S * H * d > 2 ** 32
+    w = torch.softmax(torch.randn(1, K, device=DEV, generator=g), -1)
+    q = (torch.randn(N, H, S, d, device=DEV, generator=g) * 0.5).bfloat16()
+    big = gca_hip.gca_kv_cache_indexed(q, ck, cv, ids, w, 0.125, 1.0)
+    sk, sv = ck[:, ids[0]].contiguous(), cv[:, ids[0]].contiguous()          # (1, 8, S, H*d)
+    small = gca_hip.gca_kv_cache_indexed(q, sk, sv, torch.arange(K, device=DEV)[None], w, 0.125, 1.0)
+    assert torch.equal(big, small)
+    kg = sk[0].reshape(K, S, H, d).permute(2, 0, 1, 3)[None].double().cpu()
+    vg = sv[0].reshape(K, S, H, d).permute(2, 0, 1, 3)[None].double().cpu()
+    ref = orc.gca_forward(q.double().cpu(), kg, vg, w.double().cpu(), 0.125, 1.0)
+    assert rel_err(big, ref) <= 2e-2
+    # decode steps of 1 and 2 rows on the same cache
+    for Q in (1, 2):
+        qs = q[:, :, :Q].contiguous()
+        assert torch.equal(gca_hip.gca_kv_cache_indexed(qs, ck, cv, ids, w, 0.125, 1.0),
+                           gca_hip.gca_kv_cache_indexed(qs, sk, sv, torch.arange(K, device=DEV)[None], w, 0.125, 1.0))
 
 
 def test_cfg2_indexed_equals_gathered():

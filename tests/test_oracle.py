@@ -321,6 +321,7 @@ def test_module_forward_vs_loops():
     dim = H * d
     hidden = _rand(N, C, S, dim, seed=72)
     ck, cv = _rand(N, C, S, Hkv * d, seed=73, scale=0.5), _rand(N, C, S, Hkv * d, seed=74, scale=0.5)
+    ck[:, :, -1], cv[:, :, -1] = 0, 0          # the landmark row as the model caches it (model/DRT.py:771-779)
     lq, lk = _rand(N, C, 8, seed=75), _rand(N, C, 8, seed=76)
     nw, wq, bq, wo, bo = _rand(dim, seed=77), _rand(dim, dim, seed=78, scale=0.2), _rand(dim, seed=79), \
         _rand(dim, dim, seed=80, scale=0.2), _rand(dim, seed=81)
@@ -340,11 +341,19 @@ def test_module_forward_vs_loops():
                     acc = torch.zeros(d, dtype=torch.float64)
                     for j in range(idx.shape[-1]):
                         e = idx[n, c - 1, j].item()
-                        kk_ = ck[n, e, :, hk * d:(hk + 1) * d]
-                        vv_ = cv[n, e, :, hk * d:(hk + 1) * d]
+                        # the S-1 real rows; the zeroed row adds exp(0) = 1 to the denominator and nothing else
+                        kk_ = ck[n, e, :S - 1, hk * d:(hk + 1) * d]
+                        vv_ = cv[n, e, :S - 1, hk * d:(hk + 1) * d]
                         sc = (kk_ @ qh) / math.sqrt(d)
                         p = torch.exp(sc) / (1.0 + torch.exp(sc).sum())
                         acc += w[n, c - 1, j].double() * (p @ vv_)
                     heads.append(acc)
                 ref = wo @ torch.cat(heads) + bo
                 assert (got[n, c * S + s] - ref).abs().max().item() < 1e-9
+    # sm_n itself changes nothing (inert in the reference's kernels); the functional reading on the cache
+    # without the landmark row gives the same numbers as the zeroed row does
+    again = orc.gca_module_forward(hidden, ck, cv, idx, w.double(), nw, 1e-6, wq, bq, wo, bo, H, Hkv, sm_n=0.0)
+    assert torch.equal(again, got)
+    fn = orc.gca_module_forward(hidden, ck[:, :, :S - 1], cv[:, :, :S - 1], idx, w.double(), nw, 1e-6, wq, bq, wo, bo,
+                                H, Hkv, sm_n=1.0, sm_n_functional=True)
+    assert (fn - got).abs().max().item() < 1e-12
