@@ -145,9 +145,11 @@ def test_cfg3_full_size_forward_sampled_oracle():
     needle = 4321
     direction = lk[0, needle].float()
     lk[0, needle] = (4 * direction).bfloat16()
-    lq = (torch.randn(N, C, H * d, device=DEV, generator=g) + 0.5 * direction).bfloat16()
+    # queries lean towards the needle far enough that its score (mean 2.8, std 0.5) clears the best of the 16383
+    # ordinary landmarks (about 0.5) in every row
+    lq = (torch.randn(N, C, H * d, device=DEV, generator=g) + 6.0 * direction / direction.norm()).bfloat16()
     _, indices, weights = gca_hip.landmark_retrieve(lq, lk, K, H * d)
-    assert (indices[0, needle + 1:] == needle).any(-1).all()
+    assert (indices[0, needle + 1:, 0] == needle).all()
     idx = indices[:, :-1].reshape(Z, K).contiguous()
     w = weights[:, :-1].reshape(Z, K).contiguous()
     o = gca_hip.gca_kv_cache_indexed(q, ck, cv, idx, w, 0.125, 1.0)
