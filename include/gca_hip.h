@@ -44,7 +44,8 @@ enum gca_status {
     GCA_ERR_DTYPE = 3,       /* unknown element type */
     GCA_ERR_LAUNCH = 4,      /* the HIP runtime refused a launch (wrong GPU architecture, ...) */
     GCA_ERR_WORKSPACE = 5,   /* workspace pointer NULL or too small */
-    GCA_ERR_UNSUPPORTED = 6  /* valid request this build has no kernel for */
+    GCA_ERR_UNSUPPORTED = 6, /* valid request this build has no kernel for */
+    GCA_ERR_SCRATCH_LIMIT = 7 /* lmk_score_topk_static: the request needs more than LMK_STATIC_SCRATCH_BYTES */
 };
 
 /* Which kernel family a call may use.  AUTO picks the MFMA kernels when the shape
@@ -187,6 +188,22 @@ int lmk_topk(const lmk_desc* desc, const void* scores, const void* noise, int64_
 int lmk_score_topk(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, const void* noise,
                    void* scores, int64_t* indices, float* weights,
                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* lmk_score_topk for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same selection and weights, but the (N, C, E) scores and the top-k
+ * scratch live in a static device array inside the library instead of caller buffers, so the call takes inputs and
+ * outputs only and calls no allocator.  It has no counterpart in the reference (whose retrieval allocates its
+ * score, top-k and softmax tensors through torch on every call, model/DRT.py:612-627).
+ * Limit: N*C*E scores of desc.dtype (rounded up to 256 bytes) plus lmk_topk_workspace_bytes(desc) must fit
+ * LMK_STATIC_SCRATCH_BYTES, otherwise GCA_ERR_SCRATCH_LIMIT is returned and nothing is launched; the decode steps
+ * of BASELINE config 5 (one row against 262144 landmarks, 64 rows against 1024 each) need 0.5 MiB / 0.13 MiB.
+ * Every GPU the library runs on holds its own copy of the array until the process ends.  All calls on one GPU
+ * share that copy: calls that overlap on one GPU (two streams, two host threads) race on it -- serialise them.
+ * The device to use must be current (hipSetDevice) when the call is made; the array's address on a device is
+ * looked up on the first call there.  The kernels write every scratch byte they later read, nothing is cleared. */
+#define LMK_STATIC_SCRATCH_BYTES (8u << 20)
+int lmk_score_topk_static(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, const void* noise,
+                          int64_t* indices, float* weights, void* stream);
 
 /* Bytes of scratch lmk_weights_bwd needs. */
 size_t lmk_weights_bwd_workspace_bytes(const lmk_desc* desc);

@@ -1,7 +1,18 @@
 // extern "C" surface of libgca_hip.so: argument validation and dispatch only.
+#include <mutex>
 #include "gca_common.h"
 
 using namespace gca;
+
+// ---- device-resident scratch of lmk_score_topk_static ------------------------------------------------------
+// One array per GPU, part of the library's code object (it exists from the moment the library is loaded on a
+// device until the process ends).  Host code never uses the array's name as an address: the device address
+// is looked up once per device with hipGetSymbolAddress and kept in scratch_ptr[device]; kernels get that
+// pointer as an ordinary argument.  (No "used" attribute on the array: with it the compiler keeps the device symbol
+// local to the code object and the runtime cannot find the variable the host side registered.)
+constexpr size_t SCRATCH_BYTES = LMK_STATIC_SCRATCH_BYTES;
+constexpr int MAX_DEVICES = 64;
+static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
 
 namespace {
 
@@ -44,6 +55,26 @@ int pick_path(const gca_desc& d, bool& use_mfma, bool forward) {
     return GCA_OK;
 }
 
+// device address of the current device's copy of `scratch`, looked up once per device
+void* scratch_ptr[MAX_DEVICES] = {};
+std::mutex scratch_mutex;
+
+// device address of the current device's copy of `scratch`
+int scratch_of_current_device(unsigned char** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return GCA_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) return GCA_ERR_LAUNCH;
+        scratch_ptr[dev] = ptr;
+    }
+    *out = (unsigned char*)scratch_ptr[dev];
+    return GCA_OK;
+}
+
+size_t align256(size_t x) { return (x + 255) / 256 * 256; }
+
 }  // namespace
 
 extern "C" {
@@ -59,6 +90,7 @@ const char* gca_strerror(int status) {
         case GCA_ERR_LAUNCH: return "HIP refused the kernel launch (is this a gfx950 GPU?)";
         case GCA_ERR_WORKSPACE: return "workspace missing or too small";
         case GCA_ERR_UNSUPPORTED: return "no kernel for this request";
+        case GCA_ERR_SCRATCH_LIMIT: return "request needs more than the static scratch of lmk_score_topk_static holds";
     }
     return "unknown status";
 }
@@ -152,6 +184,29 @@ int lmk_score_topk(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, c
     int rc = lmk_score(desc, lmk_q, lmk_k, scores, stream);
     if (rc != GCA_OK) return rc;
     return lmk_topk(desc, scores, noise, indices, weights, workspace, workspace_bytes, stream);
+}
+
+int lmk_score_topk_static(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, const void* noise,
+                          int64_t* indices, float* weights, void* stream) {
+    int rc = check_lmk(desc);
+    if (rc != GCA_OK) return rc;
+    if (!lmk_q || !lmk_k || !indices || !weights) return GCA_ERR_NULL;
+    // scratch layout: the (N, C, E) scores, then the segment winners of the top-k.  Both are written completely
+    // by the kernels before they are read, so nothing of an earlier call has to be cleared.
+    const size_t esz = desc->dtype == GCA_BF16 ? 2 : 4;
+    const uint64_t cap = SCRATCH_BYTES / esz;                 // no product below can overflow: every factor is <= cap
+    if ((uint64_t)desc->N > cap || (uint64_t)desc->C > cap || (uint64_t)desc->E > cap) return GCA_ERR_SCRATCH_LIMIT;
+    const uint64_t rows = (uint64_t)desc->N * (uint64_t)desc->C;
+    if (rows > cap || rows * (uint64_t)desc->E > cap) return GCA_ERR_SCRATCH_LIMIT;
+    const size_t score_bytes = align256((size_t)(rows * (uint64_t)desc->E) * esz);
+    const size_t ws_bytes = lmk_topk_ws_bytes(*desc);
+    if (score_bytes + ws_bytes > SCRATCH_BYTES) return GCA_ERR_SCRATCH_LIMIT;
+    unsigned char* base = nullptr;
+    if ((rc = scratch_of_current_device(&base)) != GCA_OK) return rc;
+    void* scores = base;
+    void* ws = base + score_bytes;
+    if ((rc = launch_lmk_score(*desc, lmk_q, lmk_k, scores, (hipStream_t)stream)) != GCA_OK) return rc;
+    return launch_lmk_topk(*desc, scores, noise, indices, weights, ws, ws_bytes, (hipStream_t)stream);
 }
 
 size_t lmk_weights_bwd_workspace_bytes(const lmk_desc* desc) {

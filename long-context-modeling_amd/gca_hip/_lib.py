@@ -21,8 +21,10 @@ GCA_OK = 0
 SYMBOLS = (
     "gca_version", "gca_strerror", "gca_fwd", "gca_bwd_workspace_bytes", "gca_bwd", "gca_fwd_indexed",
     "gca_bwd_indexed", "lmk_score", "lmk_topk_workspace_bytes", "lmk_topk", "lmk_score_topk",
-    "lmk_weights_bwd_workspace_bytes", "lmk_weights_bwd", "chunk_cache_append",
+    "lmk_weights_bwd_workspace_bytes", "lmk_weights_bwd", "chunk_cache_append", "lmk_score_topk_static",
 )
+LMK_STATIC_SCRATCH_BYTES = 8 << 20
+GCA_ERR_SCRATCH_LIMIT = 7
 CHUNK_LMK_KEEP, CHUNK_LMK_ZERO, CHUNK_LMK_DROP = 0, 1, 2
 
 
@@ -84,6 +86,8 @@ def _declare(lib):
     lib.lmk_topk.argtypes = [L, P, P, I64P, FP, P, ctypes.c_size_t, P]
     lib.lmk_score_topk.restype = ctypes.c_int
     lib.lmk_score_topk.argtypes = [L, P, P, P, P, I64P, FP, P, ctypes.c_size_t, P]
+    lib.lmk_score_topk_static.restype = ctypes.c_int
+    lib.lmk_score_topk_static.argtypes = [L, P, P, P, I64P, FP, P]
     lib.lmk_weights_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.lmk_weights_bwd_workspace_bytes.argtypes = [L]
     lib.lmk_weights_bwd.restype = ctypes.c_int

@@ -118,6 +118,28 @@ def landmark_retrieve(lmk_q, lmk_k, topk, hidden_size=None, causal=True, noise=N
     return _Retrieve.apply(lmk_q, lmk_k, topk, hidden_size, causal, noise)
 
 
+def landmark_retrieve_static(lmk_q, lmk_k, topk, out_indices, out_weights, hidden_size=None, causal=True, noise=None):
+    """Scoring + selection into caller-owned ``out_indices`` (N, C, kk) int64 / ``out_weights`` (N, C, kk) float32
+    with no device allocation at all: scores and top-k scratch stay in the library's static device array
+    (``lmk_score_topk_static``, at most ``_lib.LMK_STATIC_SCRATCH_BYTES``).  For decode loops under HIP graph
+    capture.  Inputs must already be contiguous (nothing is copied); calls on one GPU must not overlap."""
+    assert lmk_q.is_cuda and lmk_q.is_contiguous() and lmk_q.dim() == 3 and lmk_q.dtype in _DT
+    assert lmk_k.dtype == lmk_q.dtype and lmk_k.dim() == 3
+    lmk_k, rows = _dense_or_strided(lmk_k)
+    N, C, Dm = lmk_q.shape
+    E = lmk_k.shape[1]
+    kk = min(E, topk)
+    assert out_indices.shape == (N, C, kk) and out_indices.dtype == torch.int64 and out_indices.is_contiguous()
+    assert out_weights.shape == (N, C, kk) and out_weights.dtype == torch.float32 and out_weights.is_contiguous()
+    assert noise is None or (noise.shape == (N, C, E) and noise.dtype == lmk_q.dtype and noise.is_contiguous())
+    desc = _lmk_desc(lmk_q.dtype, topk, N, C, E, Dm, causal, Dm if hidden_size is None else hidden_size, rows)
+    with torch.cuda.device(lmk_q.device):
+        rc = _lib.lib().lmk_score_topk_static(ctypes.byref(desc), _ptr(lmk_q), _ptr(lmk_k), _ptr(noise),
+                                              _ptr(out_indices), _ptr(out_weights), _stream(lmk_q.device))
+    _lib.check(rc, "lmk_score_topk_static")
+    return out_indices, out_weights
+
+
 def gather_chunks(chunk_k, chunk_v, indices, weights, num_kv_heads):
     """The reference's gather + layout (model/DRT.py:198-199, :629-637, :328-332): drops the
     last retrieval row and returns k, v ((N (C-1)), Hkv, K, S, d) and weights ((N (C-1)), K).
