@@ -3,20 +3,29 @@
 
 A "step" is one GCA layer pass over one synthetic batch, everything resident in HBM:
 landmark scoring + top-k + retrieval weights, indexed forward, indexed backward
-(dq, cache-shaped dk/dv, dw).  The workload is BASELINE.json's config 2:
+(dq, cache-shaped dk/dv, dw).  The headline workload is BASELINE.json's config 2:
 B=8, H=12, d=64, L=16384 (256 chunks of 64), top-k 8, bf16, softmax-off-by-one on.
 
 Prints ONE JSON line: tokens/s of the whole step, plus
-  roofline      the slowest kernel of the step timed on its own with HIP events on the launch
-                stream, against the 8 TB/s HBM peak, with the algorithmic bytes of that kernel
-  cpu_baseline  the CPU oracle (PyTorch einsum formulation + autograd) on BASELINE.json's
-                config 1, timed on this host's cores
+  roofline      the slowest kernel of the step, timed on its own with HIP events on the launch stream,
+                against the ceiling that binds it: max(algorithmic FLOPs / MFMA peak, compulsory bytes / HBM peak)
+                divided by the measured time (<= 1 by construction).  "Compulsory" = every tensor the kernel
+                reads or writes, once.  The gather-stream byte model (every query chunk streams its K
+                retrieved chunks from HBM) is reported separately as stream_model: the indexed kernels do
+                not move those bytes (the caches absorb the K-fold re-reads), so it can exceed the peak.
+  configs       every other BASELINE.json config (1 on the GPU's fp32 path, 2 without softmax-one, 2 in the
+                gathered drop-in form the reference's model calls, 3, 4, 5a, 5b): tokens/s and the same fraction
+  cpu_baseline  the CPU oracle (PyTorch einsum formulation + autograd) on BASELINE.json's config 1, timed on
+                this host's cores
+
+--only NAME runs one workload a few times and prints its entry (for rocprofv3 runs).
 """
 import argparse
 import ctypes
 import json
 import math
 import os
+import re
 import sys
 import time
 
@@ -25,28 +34,24 @@ for _p in (ROOT, os.path.join(ROOT, "long-context-modeling_amd")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
-HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the three main kernels at config 2, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# scaled by the same counters' readings for a 1 GiB device copy (summary kept under profiles/)
-MEASURED_TRAFFIC_GB = {"gca_fwd_mfma_kernel": 1.138, "gca_bwd_dq_mfma_kernel": 1.551, "gca_bwd_dkdv2_mfma_kernel": 1.776}
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary of the config-2 step (scaled by a copy kernel of known size)
+TRAFFIC_PROFILE = os.path.join("profiles", "gca_step_cfg2_bf16.txt")
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def make_inputs(torch, dev, seed, N, C, H, S, d):
-    """Config-2 synthetic data: q, K, V ~ N(0,1)*0.5; landmark keys = per-chunk mean of K + N(0, 0.1);
-    landmark queries ~ N(0,1); grad_output ~ N(0,1)."""
-    g = torch.Generator(device=dev).manual_seed(seed)
-    Z = N * (C - 1)
-    q = (torch.randn(Z, H, S, d, device=dev, generator=g) * 0.5).bfloat16().requires_grad_(True)
-    ck = (torch.randn(N, C, S, H * d, device=dev, generator=g) * 0.5).bfloat16().requires_grad_(True)
-    cv = (torch.randn(N, C, S, H * d, device=dev, generator=g) * 0.5).bfloat16().requires_grad_(True)
-    lk = (ck.detach().float().mean(2) + 0.1 * torch.randn(N, C, H * d, device=dev, generator=g)).bfloat16()
-    lq = torch.randn(N, C, H * d, device=dev, generator=g).bfloat16()
-    do = torch.randn(Z, H, S, d, device=dev, generator=g).bfloat16()
-    return q, ck, cv, lq, lk, do
+def bound_of(flops, nbytes, seconds, dtype="bf16"):
+    """Fraction of the binding ceiling: the larger of the two floors over the measured time."""
+    t_mfma = flops / (MFMA_PEAK_TFLOPS[dtype] * 1e12)
+    t_hbm = nbytes / (HBM_PEAK_GBS * 1e9)
+    bound = "mfma" if t_mfma >= t_hbm else "hbm"
+    return {"bound": bound, "frac": round(max(t_mfma, t_hbm) / seconds, 4),
+            "algorithmic_GFLOP": round(flops / 1e9, 2), "compulsory_GB": round(nbytes / 1e9, 4),
+            "frac_of_mfma_peak": round(t_mfma / seconds, 4), "frac_of_hbm_peak": round(t_hbm / seconds, 4)}
 
 
 def event_time(torch, fn, iters, warmup=2):
@@ -60,6 +65,58 @@ def event_time(torch, fn, iters, warmup=2):
     e1.record()
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) / iters   # ms
+
+
+def measured_traffic():
+    """{kernel name: HBM GB per launch} from the tracked counter summary (lines "HBM_TRAFFIC_GB <kernel> <GB>"),
+    or {} when the file is absent."""
+    path = os.path.join(ROOT, TRAFFIC_PROFILE)
+    out = {}
+    if not os.path.exists(path):
+        return out
+    for line in open(path):
+        m = re.match(r"^HBM_TRAFFIC_GB\s+(\w+)\s+([\d.]+)\s*$", line.strip())
+        if m:
+            out[m.group(1)] = float(m.group(2))
+    return out
+
+
+# ----------------------------------------------------------------------------------------- config 2
+
+def cfg2_inputs(torch, dev, seed, N=8, C=256, H=12, S=64, d=64):
+    """Config-2 synthetic data: q, K, V ~ N(0,1)*0.5; landmark keys = per-chunk mean of K + N(0, 0.1);
+    landmark queries ~ N(0,1); grad_output ~ N(0,1)."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    Z = N * (C - 1)
+    q = (torch.randn(Z, H, S, d, device=dev, generator=g) * 0.5).bfloat16().requires_grad_(True)
+    ck = (torch.randn(N, C, S, H * d, device=dev, generator=g) * 0.5).bfloat16().requires_grad_(True)
+    cv = (torch.randn(N, C, S, H * d, device=dev, generator=g) * 0.5).bfloat16().requires_grad_(True)
+    lk = (ck.detach().float().mean(2) + 0.1 * torch.randn(N, C, H * d, device=dev, generator=g)).bfloat16()
+    lq = torch.randn(N, C, H * d, device=dev, generator=g).bfloat16()
+    do = torch.randn(Z, H, S, d, device=dev, generator=g).bfloat16()
+    return q, ck, cv, lq, lk, do
+
+
+def cfg2_work(N=8, C=256, H=12, S=64, d=64, K=8, e=2):
+    """Algorithmic FLOPs, compulsory bytes and gather-stream bytes of config 2, whole step and per kernel."""
+    Z = N * (C - 1)
+    gemm = 2 * Z * H * K * S * S * d                       # one S x S x d product per (z, head, slot)
+    q_b = Z * H * S * d * e                                 # q, o, dO, dq each
+    cache_b = N * C * S * H * d * e                         # K cache, V cache, dK, dV each
+    lse_b = Z * H * K * S * 4                               # lse, delta each
+    per_kernel = {
+        "gca_fwd_mfma_kernel": {"flops": 2 * gemm, "bytes": 2 * q_b + 2 * cache_b + lse_b},
+        "gca_bwd_dq_mfma_kernel": {"flops": 3 * gemm, "bytes": 3 * q_b + 2 * cache_b + 2 * lse_b},
+        # dk/dv: S recompute, dP, dV, dK; reads q, dO, K, V, lse, delta, writes dK, dV
+        "gca_bwd_dkdv2_mfma_kernel": {"flops": 4 * gemm, "bytes": 2 * q_b + 4 * cache_b + 2 * lse_b},
+    }
+    tokens = N * C * S
+    stream = {"gca_fwd_mfma_kernel": (2 * H * d * e + 2 * K * H * d * e + 4 * H * K) * tokens,
+              "gca_bwd_dq_mfma_kernel": (3 * H * d * e + 4 * H * K + 2 * K * H * d * e) * tokens,
+              "gca_bwd_dkdv2_mfma_kernel": (2 * K * H * d * 4) * tokens}
+    step = {"flops": 7 * gemm,                               # algorithmic: 2 fwd + 5 bwd products
+            "bytes": (2 * q_b + 2 * cache_b + lse_b) + (3 * q_b + 4 * cache_b + 3 * lse_b)}
+    return per_kernel, stream, step
 
 
 def kernel_times(torch, q, ck, cv, idx, w, do, sm_scale, sm_n, iters):
@@ -99,100 +156,199 @@ def kernel_times(torch, q, ck, cv, idx, w, do, sm_scale, sm_n, iters):
 
     fwd()
     bwd(0)()
-    times = {
+    return {
         "gca_fwd_mfma_kernel": event_time(torch, fwd, iters),
         "gca_bwd_dq_mfma_kernel": event_time(torch, bwd(1), iters),
-        "gca_list_build(3 launches)": event_time(torch, bwd(8), iters),
+        "gca_list_build": event_time(torch, bwd(8), iters),
         "gca_bwd_dkdv2_mfma_kernel": event_time(torch, bwd(2), iters),
         "gca_bwd_dkdv_reduce_kernel": event_time(torch, bwd(16), iters),
         "gca_bwd_dw_kernel": event_time(torch, bwd(4), iters),
     }
-    return times
 
 
-def other_configs(torch, dev, seed):
-    """BASELINE configs 3, 4, 5 on the same GPU: absolute tokens/s and the fraction of the binding
-    (HBM) roofline from the stream-model bytes.  Forward-only configs time scoring + top-k + forward."""
+def run_cfg2_gathered(torch, dev, seed, iters):
+    """Config 2 through the drop-in call the reference's model makes (model/DRT.py:380): attention(q, k, v, weights,
+    ...) on gathered, K-times-larger copies of the retrieved chunks, forward + backward.  Here the K-fold bytes are
+    real HBM traffic.  `with_gather` adds the reference-style gather copies (model/DRT.py:193-200, :320-332) and
+    autograd's scatter-add of dk/dv back into the cache."""
+    import gca_hip
+    N, C, H, S, d, K = 8, 256, 12, 64, 64, 8
+    q, ck, cv, lq, lk, do = cfg2_inputs(torch, dev, seed)
+    Z = N * (C - 1)
+    _, indices, weights = gca_hip.landmark_retrieve(lq, lk, K, H * d)
+    kg, vg, wg = gca_hip.gather_chunks(ck.detach(), cv.detach(), indices, weights, H)
+    kg.requires_grad_(True); vg.requires_grad_(True)
+    wg = wg.requires_grad_(True)
+
+    def step():
+        o = gca_hip.attention(q, kg, vg, wg, 0.125, 1.0)
+        return torch.autograd.grad(o, (q, kg, vg, wg), do)
+
+    def step_with_gather():
+        _, ind, wts = gca_hip.landmark_retrieve(lq, lk, K, H * d)
+        k2, v2, w2 = gca_hip.gather_chunks(ck, cv, ind, wts, H)
+        o = gca_hip.attention(q, k2, v2, w2.requires_grad_(True), 0.125, 1.0)
+        return torch.autograd.grad(o, (q, ck, cv, w2), do)
+
+    t = event_time(torch, step, iters) * 1e-3
+    t2 = event_time(torch, step_with_gather, max(2, iters // 2), 1) * 1e-3
+    tokens = N * C * S
+    gemm = 2 * Z * H * K * S * S * d
+    e = 2
+    q_b, g_b, lse_b = Z * H * S * d * e, Z * H * K * S * d * e, Z * H * K * S * 4
+    nbytes = (2 * q_b + 2 * g_b + lse_b) + (3 * q_b + 2 * g_b + 2 * lse_b) + (2 * q_b + 4 * g_b + 2 * lse_b)
+    out = {"tokens_per_s": round(tokens / t, 1), "ms": round(t * 1e3, 4)}
+    out.update(bound_of(7 * gemm, nbytes, t))
+    out["with_reference_style_gather_and_scatter"] = {"tokens_per_s": round(tokens / t2, 1), "ms": round(t2 * 1e3, 4)}
+    return out
+
+
+def run_cfg2(torch, dev, seed, sm_n, iters):
+    import gca_hip
+    N, C, H, S, d, K = 8, 256, 12, 64, 64, 8
+    q, ck, cv, lq, lk, do = cfg2_inputs(torch, dev, seed)
+    Z = N * (C - 1)
+
+    def step():
+        _, indices, weights = gca_hip.landmark_retrieve(lq, lk, K, H * d)
+        idx = indices[:, :-1].reshape(Z, -1).contiguous()
+        w = weights[:, :-1].reshape(Z, -1).contiguous().requires_grad_(True)
+        o = gca_hip.attention_indexed(q, ck, cv, idx, w, 0.125, sm_n)
+        return torch.autograd.grad(o, (q, ck, cv, w), do)
+
+    t = event_time(torch, step, iters) * 1e-3
+    _, _, work = cfg2_work()
+    out = {"tokens_per_s": round(N * C * S / t, 1), "ms": round(t * 1e3, 4)}
+    out.update(bound_of(work["flops"], work["bytes"], t))
+    return out
+
+
+# ----------------------------------------------------------------------------------------- other configs
+
+def run_cfg1_gpu(torch, dev, seed, iters):
+    """Config 1 (fp32, B=2, H=4, d=64, 16 chunks, top-k 4, softmax-one) on the GPU's fp32 kernels."""
+    import gca_hip
+    N, C, H, S, d, K = 2, 16, 4, 64, 64, 4
+    g = torch.Generator(device=dev).manual_seed(seed + 2)
+    q_all = (torch.randn(N, C, H, S, d, device=dev, generator=g) * 0.5).requires_grad_(True)
+    ck = (torch.randn(N, C, S, H * d, device=dev, generator=g) * 0.5).requires_grad_(True)
+    cv = (torch.randn(N, C, S, H * d, device=dev, generator=g) * 0.5).requires_grad_(True)
+    lq, lk = torch.randn(N, C, H * d, device=dev, generator=g), torch.randn(N, C, H * d, device=dev, generator=g)
+    do = torch.randn(N, C, H, S, d, device=dev, generator=g)
+
+    def step():
+        out, _, _ = gca_hip.gca_layer(q_all, ck, cv, lq, lk, K, sm_n=1.0)
+        return torch.autograd.grad(out, (q_all, ck, cv), do)
+
+    t = event_time(torch, step, iters, 3) * 1e-3
+    Z = N * (C - 1)
+    gemm = 2 * Z * H * K * S * S * d
+    e = 4
+    q_b, c_b, lse_b = Z * H * S * d * e, N * C * S * H * d * e, Z * H * K * S * 4
+    out = {"tokens_per_s": round(N * C * S / t, 1), "ms": round(t * 1e3, 4)}
+    out.update(bound_of(7 * gemm, 5 * q_b + 6 * c_b + 4 * lse_b, t, "fp32"))
+    out["note"] = "a handful of small launches: launch-latency bound at this size"
+    return out
+
+
+def run_cfg4(torch, dev, seed, iters):
+    """Config 4: GQA, wider heads, fwd+bwd.  Retrieval score logits ~ N(0,1) are given directly."""
     import gca_hip
     g = torch.Generator(device=dev).manual_seed(seed + 1)
+    N, C, Hq, Hkv, S, d, K = 4, 512, 32, 8, 64, 128, 16
+    Z = N * (C - 1)
 
     def rn(*shape, scale=1.0):
         return (torch.randn(*shape, device=dev, generator=g) * scale).bfloat16()
 
-    out = {}
-    # ---- config 4: GQA, wider heads, fwd+bwd.  Retrieval score logits ~ N(0,1) are given directly.
-    N, C, Hq, Hkv, S, d, K = 4, 512, 32, 8, 64, 128, 16
-    Z = N * (C - 1)
     q = rn(Z, Hq, S, d, scale=0.35).requires_grad_(True)
     do = rn(Z, Hq, S, d)
     ck = rn(N, C, S, Hkv * d, scale=0.35).requires_grad_(True)
     cv = rn(N, C, S, Hkv * d, scale=0.35).requires_grad_(True)
     scores = torch.randn(N, C, C, device=dev, generator=g).bfloat16()
 
-    def step4():
+    def step():
         indices, weights = gca_hip.landmark_topk(scores, K)
         idx = indices[:, :-1].reshape(Z, K).contiguous()
         w = weights[:, :-1].reshape(Z, K).contiguous().requires_grad_(True)
         o = gca_hip.attention_indexed(q, ck, cv, idx, w, 1.0 / math.sqrt(d), 0.0)
         return torch.autograd.grad(o, (q, ck, cv, w), do)
 
-    t = event_time(torch, step4, 5) * 1e-3
+    t = event_time(torch, step, iters) * 1e-3
     tokens = N * C * S
+    gemm = 2 * Z * Hq * K * S * S * d
     e = 2
-    nbytes = (2 * Hq * d * e + 2 * K * Hkv * d * e + 4 * Hq * K) + (3 * Hq * d * e + 4 * Hq * K + 2 * K * Hkv * d * e + 2 * K * Hkv * d * 4)
-    flops = 14 * Hq * K * S * d
-    t_roof = max(nbytes * tokens / (HBM_PEAK_GBS * 1e9), flops * tokens / 2.5e15)
-    out["cfg4_gqa_d128_fwd_bwd"] = {"tokens_per_s": round(tokens / t, 1), "ms": round(t * 1e3, 3),
-                                    "frac_of_binding_roofline": round(t_roof / t, 4), "bound": "hbm",
-                                    "algorithmic_TFLOP_per_s": round(flops * tokens / t / 1e12, 1)}
-    del q, do, ck, cv, scores
+    q_b, c_b, lse_b = Z * Hq * S * d * e, N * C * S * Hkv * d * e, Z * Hq * K * S * 4
+    out = {"tokens_per_s": round(tokens / t, 1), "ms": round(t * 1e3, 3)}
+    out.update(bound_of(7 * gemm, 5 * q_b + 6 * c_b + 4 * lse_b, t))
+    return out
 
-    # ---- config 3: 1M-token prefill, forward only, one needle chunk with a 4x landmark
+
+def run_cfg3(torch, dev, seed, iters):
+    """Config 3: 1M-token prefill, forward only, one needle chunk whose landmark has 4x norm."""
+    import gca_hip
+    g = torch.Generator(device=dev).manual_seed(seed + 3)
     N, C, H, S, d, K = 1, 16384, 12, 64, 64, 8
     Z = C - 1
+
+    def rn(*shape, scale=1.0):
+        return (torch.randn(*shape, device=dev, generator=g) * scale).bfloat16()
+
     q = rn(Z, H, S, d, scale=0.5)
     ck, cv = rn(N, C, S, H * d, scale=0.5), rn(N, C, S, H * d, scale=0.5)
     lk = (ck.float().mean(2) + 0.1 * torch.randn(N, C, H * d, device=dev, generator=g)).bfloat16()
-    lq = rn(N, C, H * d)
     needle = 4321
-    lk[0, needle] = lk[0, needle] * 4 + lq[0, -1] * 0      # 4x norm at a fixed position
-    lq = (lq + 0.5 * lk[0, needle]).bfloat16()            # queries correlate with the needle
+    direction = lk[0, needle].float()
+    lk[0, needle] = (4 * direction).bfloat16()
+    lq = (torch.randn(N, C, H * d, device=dev, generator=g) + 6.0 * direction / direction.norm()).bfloat16()
 
-    def step3():
+    def step():
         _, indices, weights = gca_hip.landmark_retrieve(lq, lk, K, H * d)
         idx = indices[:, :-1].reshape(Z, K).contiguous()
         w = weights[:, :-1].reshape(Z, K).contiguous()
         return gca_hip.gca_kv_cache_indexed(q, ck, cv, idx, w, 0.125, 1.0), indices
 
-    _, indices = step3()
+    _, indices = step()
     hit = (indices[0, needle + 1:] == needle).any(-1).float().mean().item()
-    t = event_time(torch, lambda: step3(), 3, 1) * 1e-3
+    t = event_time(torch, lambda: step(), iters, 1) * 1e-3
     tokens = N * C * S
-    nbytes = (2 * H * d * e + 2 * K * H * d * e + 4 * H * K) * tokens + 2 * N * C * H * d * e
-    out["cfg3_prefill_1M_fwd"] = {"tokens_per_s": round(tokens / t, 1), "ms": round(t * 1e3, 3),
-                                  "frac_of_binding_roofline": round(nbytes / (HBM_PEAK_GBS * 1e9) / t, 4), "bound": "hbm",
-                                  "needle_selected_by_later_rows": round(hit, 4)}
-    del q, ck, cv, lk, lq
+    e = 2
+    flops = 2 * (2 * Z * H * K * S * S * d) + C * C * H * d            # attention + the causally useful half of the scoring
+    nbytes = 2 * Z * H * S * d * e + 2 * N * C * S * H * d * e + 2 * N * C * H * d * e + 2 * C * C * e   # q, o, K, V, landmarks, scores out + in
+    out = {"tokens_per_s": round(tokens / t, 1), "ms": round(t * 1e3, 3), "needle_selected_by_later_rows": round(hit, 4)}
+    out.update(bound_of(flops, nbytes, t))
+    return out
 
-    # ---- config 5: one decode chunk (64 new tokens) per sequence against a long cache
-    for name, N, E in (("cfg5a_decode_B1_16M", 1, 262144), ("cfg5b_decode_B64_64K", 64, 1024)):
-        H, S, d, K = 12, 64, 64, 8
-        ck, cv = rn(N, E, S, H * d, scale=0.5), rn(N, E, S, H * d, scale=0.5)
-        lk, lq = rn(N, E, H * d), rn(N, 1, H * d)
-        q = rn(N, H, S, d, scale=0.5)
 
-        def step5():
-            _, indices, weights = gca_hip.landmark_retrieve(lq, lk, K, H * d)
-            return gca_hip.gca_kv_cache_indexed(q, ck, cv, indices.view(N, K), weights.view(N, K), 0.125, 1.0)
+def run_cfg5(torch, dev, seed, which, iters):
+    """Config 5: one decode chunk (64 new tokens) per sequence against a long cache: landmark scan + top-k over
+    every cached chunk, then chunk attention for the 64 query tokens."""
+    import gca_hip
+    g = torch.Generator(device=dev).manual_seed(seed + 5)
+    N, E = {"a": (1, 262144), "b": (64, 1024)}[which]
+    H, S, d, K = 12, 64, 64, 8
+    ck = torch.empty((N, E, S, H * d), device=dev, dtype=torch.bfloat16)
+    cv = torch.empty((N, E, S, H * d), device=dev, dtype=torch.bfloat16)
+    slab = max(1, (1 << 26) // (S * H * d))
+    for a in range(0, E, slab):
+        ck[:, a:a + slab].normal_(0, 0.5, generator=g)
+        cv[:, a:a + slab].normal_(0, 0.5, generator=g)
+    lk = torch.randn(N, E, H * d, device=dev, generator=g).bfloat16()
+    lq = torch.randn(N, 1, H * d, device=dev, generator=g).bfloat16()
+    q = (torch.randn(N, H, S, d, device=dev, generator=g) * 0.5).bfloat16()
 
-        t = event_time(torch, step5, 20, 3) * 1e-3
-        nbytes = N * E * H * d * e + N * (2 * K * S * H * d * e + 2 * H * S * d * e)
-        out[name] = {"new_tokens_per_s": round(N * S / t, 1), "us": round(t * 1e6, 2),
-                     "frac_of_binding_roofline": round(nbytes / (HBM_PEAK_GBS * 1e9) / t, 4), "bound": "hbm",
-                     "scan_GB_per_s": None}
-        t_scan = event_time(torch, lambda: gca_hip.landmark_scores(lq, lk, H * d), 20, 3) * 1e-3
-        out[name]["scan_GB_per_s"] = round(N * E * H * d * e / t_scan / 1e9, 1)
-        del ck, cv, lk, lq, q
+    def step():
+        _, indices, weights = gca_hip.landmark_retrieve(lq, lk, K, H * d)
+        return gca_hip.gca_kv_cache_indexed(q, ck, cv, indices.view(N, K), weights.view(N, K), 0.125, 1.0)
+
+    t = event_time(torch, step, iters, 3) * 1e-3
+    e = 2
+    nbytes = N * E * H * d * e + N * (2 * K * S * H * d * e + 2 * H * S * d * e)       # landmark scan + retrieved K/V + q, o
+    flops = 2 * N * E * H * d + 2 * (2 * N * H * K * S * S * d)
+    out = {"new_tokens_per_s": round(N * S / t, 1), "us": round(t * 1e6, 2)}
+    out.update(bound_of(flops, nbytes, t))
+    t_scan = event_time(torch, lambda: gca_hip.landmark_scores(lq, lk, H * d), iters, 3) * 1e-3
+    out["scan_GB_per_s"] = round(N * E * H * d * e / t_scan / 1e9, 1)
     return out
 
 
@@ -200,8 +356,7 @@ def cpu_baseline(torch, budget_s=12.0):
     """CPU oracle at BASELINE.json config 1 (fp32, B=2, H=4, d=64, L=1024, chunk 64, top-k 4, softmax1 on):
     retrieval + forward + autograd backward, median over the iterations that fit the budget."""
     from oracle import gca_oracle as orc
-    cores = min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(cores)
+    threads = torch.get_num_threads()          # the host's share as the environment set it (OMP_NUM_THREADS)
     torch.manual_seed(0)
     N, C, H, S, d, K = 2, 16, 4, 64, 64, 4
     q_all = (torch.randn(N, C, H, S, d) * 0.5).requires_grad_(True)
@@ -224,9 +379,35 @@ def cpu_baseline(torch, budget_s=12.0):
         ts.append(time.perf_counter() - t0)
     ts.sort()
     med = ts[len(ts) // 2]
-    return {"value": N * C * S / med, "unit": "tokens/s", "cores": cores, "kind": "port",
+    return {"value": N * C * S / med, "unit": "tokens/s", "cores": threads, "kind": "port",
             "sample": f"config 1 (fp32 B=2 H=4 d=64 L=1024 chunk=64 top-k=4), median of {len(ts)} fwd+bwd steps, "
-                      f"{med * 1e3:.2f} ms/step, torch {torch.__version__}"}
+                      f"{med * 1e3:.2f} ms/step, {threads} torch threads on a host reporting os.cpu_count()="
+                      f"{os.cpu_count()}, torch {torch.__version__}"}
+
+
+WORKLOADS = ("cfg1_fp32_gpu", "cfg2_bf16_sm0", "cfg2_bf16_gathered_dropin", "cfg3_prefill_1M_fwd", "cfg4_gqa_d128_fwd_bwd",
+             "cfg5a_decode_B1_16M", "cfg5b_decode_B64_64K")
+
+
+def run_workload(torch, dev, seed, name, quick=False):
+    torch.cuda.empty_cache()
+    if name == "cfg1_fp32_gpu":
+        return run_cfg1_gpu(torch, dev, seed, 5 if quick else 50)
+    if name == "cfg2_bf16_sm0":
+        return run_cfg2(torch, dev, seed, 0.0, 3 if quick else 10)
+    if name == "cfg2_bf16_sm1":
+        return run_cfg2(torch, dev, seed, 1.0, 3 if quick else 10)
+    if name == "cfg2_bf16_gathered_dropin":
+        return run_cfg2_gathered(torch, dev, seed, 3 if quick else 8)
+    if name == "cfg3_prefill_1M_fwd":
+        return run_cfg3(torch, dev, seed, 2 if quick else 5)
+    if name == "cfg4_gqa_d128_fwd_bwd":
+        return run_cfg4(torch, dev, seed, 2 if quick else 5)
+    if name == "cfg5a_decode_B1_16M":
+        return run_cfg5(torch, dev, seed, "a", 5 if quick else 30)
+    if name == "cfg5b_decode_B64_64K":
+        return run_cfg5(torch, dev, seed, "b", 5 if quick else 30)
+    raise SystemExit(f"bench.py: unknown workload {name}")
 
 
 def main():
@@ -237,8 +418,9 @@ def main():
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--sm-n", type=float, default=1.0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--all-configs", action="store_true",
-                    help="also time BASELINE configs 3, 4 and 5 (adds an other_configs object to the JSON line)")
+    ap.add_argument("--no-other-configs", action="store_true", help="headline workload only")
+    ap.add_argument("--only", default=None, choices=WORKLOADS + ("cfg2_bf16_sm1",),
+                    help="run just this workload a few times and print its entry (profiling runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 1 GiB device-to-device copy (a kernel of known traffic, for scaling "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
@@ -252,11 +434,22 @@ def main():
     import gca_hip
 
     dev = torch.device("cuda:0")
+    if args.copy_calibration:
+        src = torch.empty(1 << 29, device=dev, dtype=torch.bfloat16).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    if args.only:
+        print(json.dumps({args.only: run_workload(torch, dev, args.seed, args.only, quick=True)}), flush=True)
+        return
+
     N, C, H, S, d, K = 8, 256, 12, 64, 64, 8
     L_tokens = C * S
     sm_scale = 1.0 / math.sqrt(d)
     log(f"workload cfg2: B={N} H={H} d={d} L={L_tokens} chunk={S} top-k={K} bf16 sm_n={args.sm_n} seed={args.seed}")
-    q, ck, cv, lq, lk, do = make_inputs(torch, dev, args.seed, N, C, H, S, d)
+    q, ck, cv, lq, lk, do = cfg2_inputs(torch, dev, args.seed, N, C, H, S, d)
     Z = N * (C - 1)
 
     def step():
@@ -265,14 +458,6 @@ def main():
         w = weights[:, :-1].reshape(Z, -1).contiguous().requires_grad_(True)
         o = gca_hip.attention_indexed(q, ck, cv, idx, w, sm_scale, args.sm_n)
         return torch.autograd.grad(o, (q, ck, cv, w), do)
-
-    if args.copy_calibration:
-        src = torch.empty(1 << 29, device=dev, dtype=torch.bfloat16).normal_()
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
 
     for _ in range(args.warmup):
         step()
@@ -293,23 +478,32 @@ def main():
     t_retr = event_time(torch, lambda: gca_hip.landmark_retrieve(lq, lk, K, H * d), max(args.steps, 10))
     log("kernel times (ms): " + ", ".join(f"{k}={v:.3f}" for k, v in kt.items()) + f", retrieval={t_retr:.3f}")
 
-    # algorithmic bytes per token (stream model: every query chunk streams its K retrieved chunks once)
-    e = 2
-    b_fwd = 2 * H * d * e + 2 * K * H * d * e + 4 * H * K
-    b_dq = 2 * H * d * e + 4 * H * K + 2 * K * H * d * e + H * d * e          # q, dO, lse, gather, dq
-    b_dkdv = 2 * K * H * d * 4                                                # fp32 dK/dV accumulation
-    model = {"gca_fwd_mfma_kernel": b_fwd, "gca_bwd_dq_mfma_kernel": b_dq, "gca_bwd_dkdv2_mfma_kernel": b_dkdv}
-    dom = max(model, key=lambda k_: kt[k_])
-    achieved = model[dom] * tokens / (kt[dom] * 1e-3) / 1e9
-    step_bytes = (b_fwd + b_dq + b_dkdv) * tokens
-    roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": round(MEASURED_TRAFFIC_GB[dom] / (kt[dom] * 1e-3), 1),
-                "traffic_GB_per_launch": MEASURED_TRAFFIC_GB[dom],
-                "algorithmic_GB_per_launch": round(model[dom] * tokens / 1e9, 3),
+    per_kernel, stream, step_work = cfg2_work(N, C, H, S, d, K)
+    dom = max(per_kernel, key=lambda k_: kt[k_])
+    t_dom = kt[dom] * 1e-3
+    b = bound_of(per_kernel[dom]["flops"], per_kernel[dom]["bytes"], t_dom)
+    traffic = measured_traffic()
+    if b["bound"] == "mfma":
+        achieved, peak, unit = per_kernel[dom]["flops"] / t_dom / 1e12, MFMA_PEAK_TFLOPS["bf16"], "TFLOP/s"
+    else:
+        achieved, peak, unit = per_kernel[dom]["bytes"] / t_dom / 1e9, HBM_PEAK_GBS, "GB/s"
+    roofline = {"bound": b["bound"], "kernel": dom, "achieved": round(achieved, 1), "peak": peak, "unit": unit,
+                "frac": b["frac"],
+                "traffic": round(traffic[dom] * 1e9) if dom in traffic else None,
+                "traffic_unit": "HBM bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-calibrated)",
+                "traffic_source": TRAFFIC_PROFILE if dom in traffic else None,
+                "algorithmic_GFLOP_per_launch": b["algorithmic_GFLOP"], "compulsory_GB_per_launch": b["compulsory_GB"],
+                "frac_of_mfma_peak": b["frac_of_mfma_peak"], "frac_of_hbm_peak": b["frac_of_hbm_peak"],
                 "kernel_ms": {k_: round(v, 4) for k_, v in kt.items()},
-                "step_algorithmic_GB": round(step_bytes / 1e9, 3),
-                "step_frac_of_hbm_roofline": round(step_bytes / dt / 1e9 / HBM_PEAK_GBS, 4)}
+                "per_kernel_frac": {k_: bound_of(per_kernel[k_]["flops"], per_kernel[k_]["bytes"], kt[k_] * 1e-3)["frac"]
+                                    for k_ in per_kernel},
+                "step": bound_of(step_work["flops"], step_work["bytes"], dt),
+                "stream_model": {"note": "gather-stream bytes (every query chunk streams its K retrieved chunks); not a "
+                                         "ceiling for the indexed kernels, whose re-reads hit the caches",
+                                 "GB_per_launch": round(stream[dom] / 1e9, 3),
+                                 "GB_per_s": round(stream[dom] / t_dom / 1e9, 1),
+                                 "step_GB": round(sum(stream.values()) / 1e9, 3),
+                                 "step_over_hbm_peak": round(sum(stream.values()) / dt / 1e9 / HBM_PEAK_GBS, 4)}}
 
     out = {
         "metric": "GCA fwd+bwd tokens/s at L=16K (1 GPU)", "value": round(value, 1), "unit": "tokens/s",
@@ -320,10 +514,13 @@ def main():
                    "softmax_off_by_one": args.sm_n},
         "roofline": roofline,
     }
-    if args.all_configs:
-        del q, ck, cv, lq, lk, do
-        torch.cuda.empty_cache()
-        out["other_configs"] = other_configs(torch, dev, args.seed)
+    del q, ck, cv, lq, lk, do
+    if not args.no_other_configs:
+        out["configs"] = {}
+        for name in WORKLOADS:
+            t0 = time.perf_counter()
+            out["configs"][name] = run_workload(torch, dev, args.seed, name)
+            log(f"{name}: {out['configs'][name]}  ({time.perf_counter() - t0:.1f} s)")
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch)
     print(json.dumps(out), flush=True)
