@@ -142,7 +142,7 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
         sum += __shfl_xor(sum, 32);
         const float l = sum + p.sm_n * __builtin_amdgcn_exp2f(-m2);
         const float wj = load_w(w, w_is_bf16, z * p.K + j);
-        const float inv = wj / l;
+        const float inv = wj * __builtin_amdgcn_rcpf(l);      // l >= 1: the row maximum contributes exp2(0)
         if (lse != nullptr && h == 0 && row_ok)
             lse[((z * p.Hq + hq) * (int64_t)p.K + j) * p.Q_CTX + q0 + n] = m2 + __builtin_amdgcn_logf(l);
 

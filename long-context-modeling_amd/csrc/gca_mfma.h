@@ -79,13 +79,21 @@ __device__ __forceinline__ unsigned lds_offset_of(const void* lds_ptr) {
 // reserved register it will not save around the statement -- which is what is wanted here.)
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
-__device__ __forceinline__ void lds_dma_b128(const void* gptr, unsigned lds_addr) {
-    const int a = __builtin_amdgcn_readfirstlane((int)lds_addr);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(a), "v"(gptr) : "memory", "m0");
+// Address form: a wavefront-uniform 64-bit base in scalar registers plus a 32-bit unsigned byte offset per lane, so
+// issuing a copy costs no vector-ALU address arithmetic (the per-lane offsets of a tile are computed once per kernel).
+__device__ __forceinline__ const void* uniform_ptr(const void* p) {
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return (const void*)(uintptr_t)(((uint64_t)hi << 32) | lo);
 }
-__device__ __forceinline__ void lds_dma_b32(const void* gptr, unsigned lds_addr) {
+__device__ __forceinline__ void lds_dma_b128(const void* sbase, unsigned voff, unsigned lds_addr) {
     const int a = __builtin_amdgcn_readfirstlane((int)lds_addr);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(a), "v"(gptr) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(a), "v"(voff), "s"(sbase) : "memory", "m0");
+}
+__device__ __forceinline__ void lds_dma_b32(const void* sbase, unsigned voff, unsigned lds_addr) {
+    const int a = __builtin_amdgcn_readfirstlane((int)lds_addr);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(a), "v"(voff), "s"(sbase) : "memory", "m0");
 }
 #pragma clang diagnostic pop
 
@@ -103,7 +111,7 @@ struct TileLoader {
     static constexpr int NW = NT / 64;              // wavefronts sharing the copy
     static constexpr int NI = ROWS / RPI / NW;      // instructions per wavefront per tile
     static_assert(NI >= 1 && NI * RPI * NW == ROWS, "tile must split evenly over the wavefronts");
-    int goff[NI];      // element offset of this lane's piece in instruction i
+    unsigned goff[NI];      // byte offset of this lane's piece in instruction i
     int wave;
     __device__ __forceinline__ TileLoader(int tid, int rs) {
         const int lane = tid & 63;
@@ -112,19 +120,20 @@ struct TileLoader {
         for (int i = 0; i < NI; ++i) {
             const int row = (i * NW + wave) * RPI + lane / PPR;
             const int lp = (lane % PPR) ^ swz(row);
-            goff[i] = row * rs + lp * 8;
+            goff[i] = (unsigned)(row * rs + lp * 8) * 2u;
         }
     }
     __device__ __forceinline__ void issue(const uint16_t* tile, unsigned char* lds_tile) const {
         const unsigned base = lds_offset_of(lds_tile) + wave * 1024;
+        const void* sb = uniform_ptr(tile);          // the tile's first element: the same for every lane
 #pragma unroll
-        for (int i = 0; i < NI; ++i) lds_dma_b128(tile + goff[i], base + i * NW * 1024);
+        for (int i = 0; i < NI; ++i) lds_dma_b128(sb, goff[i], base + i * NW * 1024);
     }
 };
 
 // 64 floats -> LDS (one wavefront, lane l writes element l)
 __device__ __forceinline__ void async_row64(const float* src, float* lds_dst, int lane) {
-    lds_dma_b32(src + lane, lds_offset_of(lds_dst));
+    lds_dma_b32(uniform_ptr(src), (unsigned)lane * 4u, lds_offset_of(lds_dst));
 }
 
 // all outstanding global_load_lds of this wavefront have landed (vmcnt = 0; other counters untouched)

@@ -200,24 +200,30 @@ lmk_score_mfma_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const uint16_
         }
         return;
     }
-    // async copy plan: instruction i of this wavefront fills rows (i*4 + wave)*8 .. +7 of a sub-tile
-    int64_t aoff[2], b0off[2], b1off[2];
+    // async copy plan: instruction i of this wavefront fills rows (i*4 + wave)*8 .. +7 of a sub-tile.  Scalar base
+    // (first row of the block) + per-lane 32-bit byte offset; tail rows re-read the block's last valid row.
+    unsigned aoff[2], b0off[2], b1off[2];
+    const int64_t crows = min((int64_t)64, d.C - c0), erows = d.E - e0;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const int row = (i * 4 + wave) * 8 + lane / 8;
         const int lp = (lane % 8) ^ swz(row);
-        aoff[i] = (nb * d.C + min(c0 + row, d.C - 1)) * d.Dm + lp * 8;          // tail rows re-read the last row
-        b0off[i] = (nb * d.lmk_k_rows + min(e0 + row, d.E - 1)) * d.Dm + lp * 8;
-        b1off[i] = (nb * d.lmk_k_rows + min(e0 + 64 + row, d.E - 1)) * d.Dm + lp * 8;
+        aoff[i] = (unsigned)((min((int64_t)row, crows - 1)) * d.Dm + lp * 8) * 2u;
+        b0off[i] = (unsigned)((min((int64_t)row, erows - 1)) * d.Dm + lp * 8) * 2u;
+        b1off[i] = (unsigned)((min((int64_t)row + 64, erows - 1)) * d.Dm + lp * 8) * 2u;
     }
+    const uint16_t* abase = lq + (nb * d.C + c0) * d.Dm;
+    const uint16_t* bbase = lk + (nb * d.lmk_k_rows + e0) * d.Dm;
     auto issue = [&](int k0, int buf) {
         const unsigned base = lds_offset_of(smem + buf * BUF) + wave * 1024;
+        const void* sa = uniform_ptr(abase + k0);
+        const void* sb = uniform_ptr(bbase + k0);
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const unsigned lo = base + i * 4 * 1024;
-            lds_dma_b128(lq + aoff[i] + k0, lo);
-            lds_dma_b128(lk + b0off[i] + k0, lo + TILE);
-            lds_dma_b128(lk + b1off[i] + k0, lo + 2 * TILE);
+            lds_dma_b128(sa, aoff[i], lo);
+            lds_dma_b128(sb, b0off[i], lo + TILE);
+            lds_dma_b128(sb, b1off[i], lo + 2 * TILE);
         }
     };
     f32x16 acc[2];
