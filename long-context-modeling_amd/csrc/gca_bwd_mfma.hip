@@ -200,6 +200,18 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
 // all four products for them itself (S, dP over all 64 query rows of a unit, then dV, dK), so the only
 // thing the wavefronts share is the Q / dO tile in LDS and there is one barrier per unit.  With
 // D == 128 its accumulators and operands need ~450 registers; the four-wavefront kernel below halves that.
+//
+// The element-wise work is the bottleneck of this kernel (one exp2, one product and two roundings per score on
+// the vector ALUs against four matrix products), so everything that can be moved into the matrix products is:
+//   * the stationary operands are pre-scaled once per workgroup: K' = bf16(sm_scale log2(e) K), V' = bf16(sm_scale V);
+//   * the per-query biases ride in one extra 16-wide reduction step whose B operand is the constant (1, 1, 0, ...)
+//     and whose A operand holds the bias split into two bf16 values (hi + lo, error < 2^-17 of the bias):
+//       S''  = Q K'^T  + (log2|w| - lse[q])        ->  P~ = exp2(S'')             (= |w| P)
+//       dP'' = dO V'^T + (-sm_scale delta[q])      ->  dS = P~ dP''               (= |w| sm_scale P (dP - D))
+//     so the element loop is exp2, multiply, round, round, with no bias reads from LDS.
+// Operand fetch is software-pipelined by hand: every LDS read is issued one phase (a block of matrix products or
+// the element loop) before its first use, and the barrier that hands a tile buffer back for refilling sits in the
+// middle of a unit, after the unit's last LDS read has landed, so the copies run two units ahead.
 template <int D, bool INDEXED>
 __global__ void __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2)))
 gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
@@ -211,8 +223,7 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
     constexpr int KS = D / 16, DB = D / 32;
     constexpr int RB = D * 2, TILE = 64 * RB, BUF = 2 * TILE;   // Q tile then dO tile
     __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * BUF];
-    // per wavefront and buffer: the unit's lse / delta rows, rewritten in place at the start of the unit into the
-    // exponent bias log2(w) - lse and -sm_scale * delta, so the element loop needs no per-element sub / mul for them
+    // per wavefront and buffer: the unit's lse / delta rows (64 floats each)
     __shared__ __attribute__((aligned(256))) float s_lse[2][2][64];
     __shared__ __attribute__((aligned(256))) float s_dl[2][2][64];
 
@@ -270,23 +281,33 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
         vt = v + out_off;
     }
 
-    // K, V rows of this wavefront as B operands: lane holds key 32*kbw + n, dims 16*ks + 8*h .. +7
+    // K', V' rows of this wavefront as B operands: lane holds key 32*kbw + n, dims 16*ks + 8*h .. +7
+    const float c = p.sm_scale * LOG2E;
     bf16x8 kB[KS], vB[KS];
     {
         const int64_t off = (int64_t)(32 * kbw + n) * rs + 8 * h;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            kB[ks] = *reinterpret_cast<const bf16x8*>(kt + off + 16 * ks);
-            vB[ks] = *reinterpret_cast<const bf16x8*>(vt + off + 16 * ks);
+            const bf16x8 kr = *reinterpret_cast<const bf16x8*>(kt + off + 16 * ks);
+            const bf16x8 vr = *reinterpret_cast<const bf16x8*>(vt + off + 16 * ks);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                kB[ks][e] = (__bf16)((float)kr[e] * c);
+                vB[ks][e] = (__bf16)((float)vr[e] * p.sm_scale);
+            }
         }
     }
+    // B operand of the bias step: slots 0 and 1 are one (the A operand of lanes with h == 1 is all zero)
+    bf16x8 onesB = {0, 0, 0, 0, 0, 0, 0, 0};
+    onesB[0] = (__bf16)1.0f;
+    onesB[1] = (__bf16)1.0f;
+
     f32x16 dkacc[DB], dvacc[DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
 
-    const float c = p.sm_scale * LOG2E;
     const TileLoader<D, NT> loader(tid, (int)p.q_rs);
 
     // unit u = (reference, query head of the group, 64-row query tile), tile fastest
@@ -306,7 +327,7 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
         }
     };
 
-    // asynchronous copy of unit u's Q / dO tiles and lse / delta rows into buffer `buf`
+    // asynchronous copy of unit u's Q / dO tiles and lse / delta rows into buffer `buf`; returns the unit's weight
     auto issue_unit = [&](int u, int buf) -> float {
         int64_t z; int j, hq, qrow0;
         unit_coords(u, z, j, hq, qrow0);
@@ -320,79 +341,117 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
         return load_w(w, w_is_bf16, z * p.K + j);
     };
 
-    float w_cur = issue_unit(0, 0), w_next = 0.f;
-    wait_async_tiles();
-    __syncthreads();
-
     const TrLane tr(lane);
     const int fsw = swz(n);
 
+    // ---- operand fetch helpers (LDS -> registers)
+    // A operands of S and dP for 32 query rows: lane holds query 32*qt + n, dims 16*ks + 8*h .. +7
+    auto load_rows = [&](int buf, int qt, bf16x8 (&aq)[KS], bf16x8 (&ad)[KS]) {
+        const unsigned char* qbuf = smem + buf * BUF;
+        const int rowoff = (32 * qt + n) * RB;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int po = rowoff + (((2 * ks + h) ^ fsw) << 4);
+            aq[ks] = lds_read_b128(qbuf + po);
+            ad[ks] = lds_read_b128(qbuf + TILE + po);
+        }
+    };
+    // transposed B operands of dV and dK for 32 query rows (two 16-query reduction steps x DB dim blocks)
+    auto load_cols = [&](int buf, int qt, bf16x8 (&bdo)[2][DB], bf16x8 (&bq)[2][DB]) {
+        const unsigned char* qbuf = smem + buf * BUF;
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const int o0 = tr.off(2 * qt + t2, db, RB);
+                bdo[t2][db] = lds_read_tr_pair(qbuf + TILE + o0, qbuf + TILE + o0 + 8 * RB);
+                bq[t2][db] = lds_read_tr_pair(qbuf + o0, qbuf + o0 + 8 * RB);
+            }
+    };
+    // bias as the A operand of the extra reduction step: (hi, lo, 0, ...) in lanes with h == 0, zero elsewhere
+    auto bias_operand = [&](float x) -> bf16x8 {
+        const __bf16 hi = (__bf16)x;
+        const __bf16 lo = (__bf16)(x - (float)hi);
+        bf16x8 a = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (h == 0) { a[0] = hi; a[1] = lo; }
+        return a;
+    };
+
+    // ---- prologue: unit 0 lands, unit 1 is requested, unit 0's first operands are fetched
+    float w_cur = issue_unit(0, 0), w_n1 = 0.f, w_n2 = 0.f;
+    wait_async_tiles();
+    __syncthreads();
+    if (nunits > 1) w_n1 = issue_unit(1, 1);
+    bf16x8 aq[KS], ad[KS];
+    float ls[2], dl[2];               // lse / delta of queries n and 32 + n
+    load_rows(0, 0, aq, ad);
+    ls[0] = s_lse[kbw][0][n]; ls[1] = s_lse[kbw][0][32 + n];
+    dl[0] = s_dl[kbw][0][n];  dl[1] = s_dl[kbw][0][32 + n];
+
     for (int u = 0; u < nunits; ++u) {
         const int buf = u & 1;
-        const bool more = (u + 1 < nunits);
-        if (more) w_next = issue_unit(u + 1, buf ^ 1);   // that buffer was last read in iteration u-1
-        const unsigned char* qbuf = smem + buf * BUF;
-        const unsigned char* dobuf = qbuf + TILE;
-        // |w| rides in the exponent (P~ = exp2(c S - lse + log2 |w|)), the sign of w goes on the rounded operands;
-        // a slot of weight 0 adds nothing to dk, dv
-        const float lw = __builtin_amdgcn_logf(fabsf(w_cur));
+        // |w| rides in the bias (log2 |w| - lse), the sign of w goes on the rounded operands; weight 0 -> P~ = 0
+        const float aw = fabsf(w_cur);
+        const float lw = aw > 0.f ? __builtin_amdgcn_logf(aw) : -1e30f;
         const bool wneg = w_cur < 0.f;
 
-        if (w_cur != 0.f) {
-        // this wavefront's copy of the rows: lse -> log2(w) - lse, delta -> -sm_scale * delta (LDS keeps a
-        // wavefront's own write and later reads in order, no barrier needed)
-        s_lse[kbw][buf][lane] = lw - s_lse[kbw][buf][lane];
-        s_dl[kbw][buf][lane] = -p.sm_scale * s_dl[kbw][buf][lane];
+        bf16x8 pA[2], dsA[2];
+        bf16x8 bdo[2][DB], bq[2][DB];
 #pragma unroll
         for (int qt = 0; qt < 2; ++qt) {
-            // S = Q K^T, dP = dO V^T for 32 query rows: queries in registers, key n in the lane
+            // ---- S'' and dP'' for 32 query rows: queries in registers, key n in the lane
+            const bf16x8 bs = bias_operand(lw - ls[qt]);
+            const bf16x8 bd = bias_operand(-p.sm_scale * dl[qt]);
             f32x16 s, dp;
 #pragma unroll
             for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
-            const int rowoff = (32 * qt + n) * RB;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const int po = rowoff + (((2 * ks + h) ^ fsw) << 4);
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(qbuf + po), kB[ks], s, 0, 0, 0);
-                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(dobuf + po), vB[ks], dp, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq[ks], kB[ks], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ad[ks], vB[ks], dp, 0, 0, 0);
             }
-            bf16x8 pA[2], dsA[2];
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bs, onesB, s, 0, 0, 0);
+            dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bd, onesB, dp, 0, 0, 0);
+            // fetch what the next phases need while the products run: the transposed operands of this half and
+            // the row operands of the next half
+            load_cols(buf, qt, bdo, bq);
+            if (qt == 0) load_rows(buf, 1, aq, ad);
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- element loop: registers 0..15 are queries 32*qt + 8*(r/4) + 4*h + r%4
 #pragma unroll
-            for (int a = 0; a < 4; ++a) {
-                // registers 4a .. 4a+3 are queries 32*qt + 8a + 4h + 0..3
-                f32x4 l4 = *reinterpret_cast<const f32x4*>(&s_lse[kbw][buf][32 * qt + 8 * a + 4 * h]);
-                f32x4 d4 = *reinterpret_cast<const f32x4*>(&s_dl[kbw][buf][32 * qt + 8 * a + 4 * h]);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int r = 4 * a + e;
-                    const float pw = __builtin_amdgcn_exp2f(fmaf(s[r], c, l4[e]));
-                    pA[r >> 3][r & 7] = (__bf16)pw;
-                    dsA[r >> 3][r & 7] = (__bf16)(pw * fmaf(dp[r], p.sm_scale, d4[e]));
-                }
+            for (int r = 0; r < 16; ++r) {
+                const float pw = __builtin_amdgcn_exp2f(s[r]);
+                pA[r >> 3][r & 7] = (__bf16)pw;
+                dsA[r >> 3][r & 7] = (__bf16)(pw * dp[r]);
             }
             if (wneg) {
 #pragma unroll
                 for (int t2 = 0; t2 < 2; ++t2) { pA[t2] = negate_bf16x8(pA[t2]); dsA[t2] = negate_bf16x8(dsA[t2]); }
             }
-            // dV += P~^T dO, dK += dS^T Q over these 32 queries (two 16-query reduction steps)
+            if (qt == 1) {
+                // Every LDS read of this unit has landed: hand the buffer back, request the unit after next,
+                // and fetch the first operands of the next unit, all under the last block of products.
+                __builtin_amdgcn_s_waitcnt(0x0070);        // vmcnt(0): unit u+1 has landed; lgkmcnt(0): reads done
+                __syncthreads();
+                if (u + 2 < nunits) w_n2 = issue_unit(u + 2, buf);
+                if (u + 1 < nunits) {
+                    load_rows(buf ^ 1, 0, aq, ad);
+                    ls[0] = s_lse[kbw][buf ^ 1][n]; ls[1] = s_lse[kbw][buf ^ 1][32 + n];
+                    dl[0] = s_dl[kbw][buf ^ 1][n];  dl[1] = s_dl[kbw][buf ^ 1][32 + n];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // ---- dV += P~^T dO, dK += dS^T Q over these 32 queries (two 16-query reduction steps)
 #pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2) {
-                const int t4 = 2 * qt + t2;
+            for (int t2 = 0; t2 < 2; ++t2)
 #pragma unroll
                 for (int db = 0; db < DB; ++db) {
-                    const int o0 = tr.off(t4, db, RB);
-                    const bf16x8 bdo = lds_read_tr_pair(dobuf + o0, dobuf + o0 + 8 * RB);
-                    dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pA[t2], bdo, dvacc[db], 0, 0, 0);
-                    const bf16x8 bq = lds_read_tr_pair(qbuf + o0, qbuf + o0 + 8 * RB);
-                    dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsA[t2], bq, dkacc[db], 0, 0, 0);
+                    dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pA[t2], bdo[t2][db], dvacc[db], 0, 0, 0);
+                    dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsA[t2], bq[t2][db], dkacc[db], 0, 0, 0);
                 }
-            }
         }
-        }
-
-        w_cur = w_next;
-        wait_async_tiles();
-        __syncthreads();
+        w_cur = w_n1;
+        w_n1 = w_n2;
     }
 
     // ---- write the tile: register r of block db is key row 32*kbw + 8*(r/4) + 4*h + r%4, column 32*db + n
