@@ -273,8 +273,9 @@ static int launch_d(const Params& p, const void* q, const void* k, const void* v
     ListWs ws = {};
     if (p.indexed) {
         // every chunk's list is walked whole by one workgroup here: no segments, no partial slots
-        ws = list_carve(p, GENERIC_SEG_MAX, (char*)delta + delta_bytes(p));
-        const int rc = (p.stages & GCA_STAGE_LISTS) ? list_build(p, GENERIC_SEG_MAX, idx, ws, s) : GCA_OK;
+        char* tables = (char*)delta + delta_bytes(p);
+        ws = list_carve(p, GENERIC_SEG_MAX, 1, tables, tables + list_table_bytes(p, GENERIC_SEG_MAX, 1));
+        const int rc = (p.stages & GCA_STAGE_LISTS) ? list_build(p, GENERIC_SEG_MAX, 1, idx, ws, s) : GCA_OK;
         if (rc != GCA_OK) return rc;
         if (p.stages & GCA_STAGE_DKDV)
         hipLaunchKernelGGL((gca_bwd_dkdv_generic_kernel<T, WT, D, true>), dim3((unsigned)b2), dim3(256), 0, s, p,

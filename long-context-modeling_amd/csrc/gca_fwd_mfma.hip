@@ -21,8 +21,9 @@
 //                   with lane ^ 32.
 //   P~  = w_j exp2(c S - m) / l  rounded to bf16.  Its register layout already IS the A operand of
 //                   the second product (reduction index permuted the same way on both operands).
-//   O  += P~ V_j    B = V read from LDS with ds_read_tr16_b64, which hands each lane one dim
-//                   column of a 4-key x 16-dim patch, i.e. the transposed access V needs.
+//   O^T += V_j^T P~^T  A = V read from LDS with ds_read_tr16_b64, which hands each lane one dim column of a
+//                   4-key x 16-dim patch, i.e. the transposed access V needs.  Accumulating the transpose puts the
+//                   lane's own query row into every accumulator register: the output row leaves in 8-byte stores.
 // The softmax denominator includes sm_n * exp2(-m) (sm_n virtual keys of logit 0 and value 0).
 // lse[z, h, j, row] = m + log2(l) in the log2-scaled domain, written when lse != NULL.
 #include "gca_mfma.h"
@@ -163,7 +164,8 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
             for (int db = 0; db < DB; ++db) {
                 const int o0 = tr.off(t4, db, RB);
                 const bf16x8 b = lds_read_tr_pair(vb + o0, vb + o0 + 8 * RB);
-                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pA[t4], b, oacc[db], 0, 0, 0);
+                // operands in the order (V^T, P~^T): the result is O^T, the lane's own query in every register
+                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, pA[t4], oacc[db], 0, 0, 0);
             }
         }
 
@@ -176,19 +178,20 @@ gca_fwd_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __
         }
     }
 
-    // ---- store O: register r of block db is row 8*(r/4) + 4*h + r%4, column 32*db + n
-    //      = a wavefront-uniform base per (r, db) plus one 32-bit lane offset
-    uint16_t* op = o + q_base_n(p, nseq, z, hq) + q0 * qrs;
-    const unsigned lane_off = (unsigned)(4 * h * qrs + n);
+    // ---- store O: the accumulators hold O^T -- lane (n, h) owns query row q0 + n, and registers 4a .. 4a+3 of
+    //      block db are its dims 32*db + 8a + 4h + 0..3: four consecutive bf16 = one 8-byte store
+    if (row_ok) {
+        uint16_t* op = o + q_base_n(p, nseq, z, hq) + (int64_t)(q0 + n) * qrs + 4 * h;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+        for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int row = 8 * (r >> 2) + 4 * h + (r & 3);
-            const __bf16 ob = (__bf16)oacc[db][r];
-            uint16_t* rowp = op + ((8 * (r >> 2) + (r & 3)) * qrs + 32 * db);
-            if (q0 + row < p.Q_CTX) rowp[lane_off] = __builtin_bit_cast(uint16_t, ob);
-        }
+            for (int a = 0; a < 4; ++a) {
+                union { __bf16 b[4]; uint64_t u; } pk;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) pk.b[e] = (__bf16)oacc[db][4 * a + e];
+                *reinterpret_cast<uint64_t*>(op + 32 * db + 8 * a) = pk.u;
+            }
+    }
 }
 
 bool mfma_fwd_supported(const gca_desc& d) {

@@ -111,23 +111,30 @@ struct TileLoader {
     static constexpr int NW = NT / 64;              // wavefronts sharing the copy
     static constexpr int NI = ROWS / RPI / NW;      // instructions per wavefront per tile
     static_assert(NI >= 1 && NI * RPI * NW == ROWS, "tile must split evenly over the wavefronts");
-    unsigned goff[NI];      // byte offset of this lane's piece in instruction i
+    // Instruction i of this wavefront fills rows (i*NW + wave)*RPI .. +RPI-1.  swz(row) depends on row % 8 only and
+    // (i*NW + wave)*RPI is a multiple of 8 (RPI == 8), or of 4 with the parity of wave (RPI == 4, NW even), so the
+    // lane's swizzled piece is the same in every instruction: one per-lane byte offset serves the whole tile and the
+    // step from instruction to instruction goes on the scalar base.
+    static_assert((RPI == 8 || (RPI == 4 && NW % 2 == 0)), "swizzle must not depend on the instruction index");
+    unsigned goff;          // byte offset of this lane's piece in instruction 0
+    unsigned istep;         // bytes between the rows of consecutive instructions (wavefront-uniform)
     int wave;
     __device__ __forceinline__ TileLoader(int tid, int rs) {
         const int lane = tid & 63;
         wave = tid >> 6;
-#pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const int row = (i * NW + wave) * RPI + lane / PPR;
-            const int lp = (lane % PPR) ^ swz(row);
-            goff[i] = (unsigned)(row * rs + lp * 8) * 2u;
-        }
+        const int row = wave * RPI + lane / PPR;
+        const int lp = (lane % PPR) ^ swz(row);
+        goff = (unsigned)(row * rs + lp * 8) * 2u;
+        istep = (unsigned)(NW * RPI * rs) * 2u;
     }
     __device__ __forceinline__ void issue(const uint16_t* tile, unsigned char* lds_tile) const {
         const unsigned base = lds_offset_of(lds_tile) + wave * 1024;
-        const void* sb = uniform_ptr(tile);          // the tile's first element: the same for every lane
 #pragma unroll
-        for (int i = 0; i < NI; ++i) lds_dma_b128(sb, goff[i], base + i * NW * 1024);
+        for (int i = 0; i < NI; ++i) {
+            // the rows of instruction i start i * istep bytes after the tile's first element
+            const void* sb = uniform_ptr((const unsigned char*)tile + (size_t)i * istep);
+            lds_dma_b128(sb, goff, base + i * NW * 1024);
+        }
     }
 };
 
