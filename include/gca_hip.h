@@ -16,7 +16,9 @@
  * Tensor layouts (element type T = desc.dtype; all contiguous):
  *   q, o, do, dq      (Z, Hq, Q_CTX, D)              or token-major, see gca_q_layout
  *   k, v, dk, dv      (Z, Hkv, K, K_CTX, D)          gathered ("retrieved chunks") form
- *   weights           (Z, K)      type desc.w_dtype  shared by all heads
+ *   weights           (Z, K)      type desc.w_dtype  shared by all heads; any sign.  bf16 weights are read
+ *                                                    in aligned 4-byte words: the buffer must be readable
+ *                                                    up to the next multiple of 4 bytes
  *   lse               (Z, Hq, K, Q_CTX)  float       log2 of the softmax denominator of the
  *                                                    log2-scaled scores, per retrieved chunk
  *   dw                (Z, K)      float
@@ -165,6 +167,21 @@ int gca_bwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, co
                     const int64_t* indices, const void* weights, const void* dout, const float* lse,
                     void* dq, void* dk_cache, void* dv_cache, float* dw,
                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* The reference lists gca_bwd_indexed derives from `indices` (which query chunks retrieved each cache chunk, in a
+ * fixed order) depend on the retrieval only, not on a layer's tensors.  A model whose layer group shares one
+ * retrieval (model/DRT.py:816-824 runs it once per group, :853-886 uses it in every layer of the group) builds them
+ * once with gca_lists_build and hands them to every layer's backward through gca_bwd_indexed_lists; with
+ * lists == NULL that call builds them itself, exactly like gca_bwd_indexed.  `lists` must come from a build with the
+ * same descriptor shape (dtype, Z, K, N, C, D, Q_CTX, path) and the same indices; it is only read by the backward.
+ * The build is one pass over the Z*K references (independent of the number of chunks per sequence) and
+ * deterministic.  No counterpart in the reference, where autograd re-derives the scatter for every layer. */
+size_t gca_lists_workspace_bytes(const gca_desc* desc);
+int gca_lists_build(const gca_desc* desc, const int64_t* indices, void* lists, size_t lists_bytes, void* stream);
+int gca_bwd_indexed_lists(const gca_desc* desc, const void* q, const void* k_cache, const void* v_cache,
+                          const int64_t* indices, const void* weights, const void* dout, const float* lse,
+                          void* dq, void* dk_cache, void* dv_cache, float* dw,
+                          void* workspace, size_t workspace_bytes, const void* lists, size_t lists_bytes, void* stream);
 
 /* scores[n, c, e] = <lmk_q[n, c, :], lmk_k[n, e, :]> / sqrt(hidden_size), -inf where masked.
  * lmk_q (N, C, Dm), lmk_k (N, E, Dm), scores (N, C, E), all of desc.dtype.

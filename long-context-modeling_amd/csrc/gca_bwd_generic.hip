@@ -260,7 +260,7 @@ int launch_dw(const Params& p, const float* delta, float* dw, hipStream_t s) {
 template <typename T, typename WT, int D>
 static int launch_d(const Params& p, const void* q, const void* k, const void* v, const int64_t* idx,
                     const void* w, const void* dout, const float* lse, void* dq, void* dk, void* dv,
-                    float* dw, float* delta, hipStream_t s) {
+                    float* dw, float* delta, void* lists, hipStream_t s) {
     const int nqb = (p.Q_CTX + 31) / 32;
     const int64_t b1 = p.Z * p.Hq * nqb;
     const int nkb = (p.K_CTX + 31) / 32;
@@ -274,8 +274,8 @@ static int launch_d(const Params& p, const void* q, const void* k, const void* v
     if (p.indexed) {
         // every chunk's list is walked whole by one workgroup here: no segments, no partial slots
         char* tables = (char*)delta + delta_bytes(p);
-        ws = list_carve(p, GENERIC_SEG_MAX, 1, tables, tables + list_table_bytes(p, GENERIC_SEG_MAX, 1));
-        const int rc = (p.stages & GCA_STAGE_LISTS) ? list_build(p, GENERIC_SEG_MAX, 1, idx, ws, s) : GCA_OK;
+        ws = list_carve(p, GENERIC_SEG_MAX, lists != nullptr ? lists : tables, tables + list_table_bytes(p, GENERIC_SEG_MAX));
+        const int rc = (lists == nullptr && (p.stages & GCA_STAGE_LISTS)) ? list_build(p, GENERIC_SEG_MAX, idx, ws, s) : GCA_OK;
         if (rc != GCA_OK) return rc;
         if (p.stages & GCA_STAGE_DKDV)
         hipLaunchKernelGGL((gca_bwd_dkdv_generic_kernel<T, WT, D, true>), dim3((unsigned)b2), dim3(256), 0, s, p,
@@ -293,29 +293,29 @@ static int launch_d(const Params& p, const void* q, const void* k, const void* v
 template <typename T, typename WT>
 static int launch_t(const Params& p, const void* q, const void* k, const void* v, const int64_t* idx,
                     const void* w, const void* dout, const float* lse, void* dq, void* dk, void* dv,
-                    float* dw, float* delta, hipStream_t s) {
+                    float* dw, float* delta, void* lists, hipStream_t s) {
     switch (p.D) {
-        case 16: return launch_d<T, WT, 16>(p, q, k, v, idx, w, dout, lse, dq, dk, dv, dw, delta, s);
-        case 32: return launch_d<T, WT, 32>(p, q, k, v, idx, w, dout, lse, dq, dk, dv, dw, delta, s);
-        case 64: return launch_d<T, WT, 64>(p, q, k, v, idx, w, dout, lse, dq, dk, dv, dw, delta, s);
-        case 128: return launch_d<T, WT, 128>(p, q, k, v, idx, w, dout, lse, dq, dk, dv, dw, delta, s);
-        case 256: return launch_d<T, WT, 256>(p, q, k, v, idx, w, dout, lse, dq, dk, dv, dw, delta, s);
+        case 16: return launch_d<T, WT, 16>(p, q, k, v, idx, w, dout, lse, dq, dk, dv, dw, delta, lists, s);
+        case 32: return launch_d<T, WT, 32>(p, q, k, v, idx, w, dout, lse, dq, dk, dv, dw, delta, lists, s);
+        case 64: return launch_d<T, WT, 64>(p, q, k, v, idx, w, dout, lse, dq, dk, dv, dw, delta, lists, s);
+        case 128: return launch_d<T, WT, 128>(p, q, k, v, idx, w, dout, lse, dq, dk, dv, dw, delta, lists, s);
+        case 256: return launch_d<T, WT, 256>(p, q, k, v, idx, w, dout, lse, dq, dk, dv, dw, delta, lists, s);
     }
     return GCA_ERR_SHAPE;
 }
 
 int launch_bwd_generic(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v,
                        const int64_t* indices, const void* w, const void* dout, const float* lse,
-                       void* dq, void* dk, void* dv, float* dw, float* delta, hipStream_t s) {
+                       void* dq, void* dk, void* dv, float* dw, float* delta, void* lists, hipStream_t s) {
     const Params p = make_params(d, indexed);
     if (d.dtype == GCA_F32 && d.w_dtype == GCA_F32)
-        return launch_t<float, float>(p, q, k, v, indices, w, dout, lse, dq, dk, dv, dw, delta, s);
+        return launch_t<float, float>(p, q, k, v, indices, w, dout, lse, dq, dk, dv, dw, delta, lists, s);
     if (d.dtype == GCA_F32 && d.w_dtype == GCA_BF16)
-        return launch_t<float, bf16_t>(p, q, k, v, indices, w, dout, lse, dq, dk, dv, dw, delta, s);
+        return launch_t<float, bf16_t>(p, q, k, v, indices, w, dout, lse, dq, dk, dv, dw, delta, lists, s);
     if (d.dtype == GCA_BF16 && d.w_dtype == GCA_F32)
-        return launch_t<bf16_t, float>(p, q, k, v, indices, w, dout, lse, dq, dk, dv, dw, delta, s);
+        return launch_t<bf16_t, float>(p, q, k, v, indices, w, dout, lse, dq, dk, dv, dw, delta, lists, s);
     if (d.dtype == GCA_BF16 && d.w_dtype == GCA_BF16)
-        return launch_t<bf16_t, bf16_t>(p, q, k, v, indices, w, dout, lse, dq, dk, dv, dw, delta, s);
+        return launch_t<bf16_t, bf16_t>(p, q, k, v, indices, w, dout, lse, dq, dk, dv, dw, delta, lists, s);
     return GCA_ERR_DTYPE;
 }
 

@@ -36,10 +36,6 @@ namespace gca {
 
 // references per dkdv workgroup in the indexed form: longer lists are cut into segments of this many
 constexpr int SEG_MAX = 32;
-#ifndef GCA_USE_STREAM
-#define GCA_USE_STREAM 0
-#endif
-constexpr bool USE_STREAM = GCA_USE_STREAM != 0;
 
 // ------------------------------------------------------------------------------------------- dq
 
@@ -478,325 +474,29 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
                 part[64 * D + row * D + 32 * db] = dvacc[db][r];
             }
     } else {
-        uint16_t* dkp = (uint16_t*)dk_out + out_off + (int64_t)(32 * kbw) * rs + n;
-        uint16_t* dvp = (uint16_t*)dv_out + out_off + (int64_t)(32 * kbw) * rs + n;
+        // Through LDS, so that the rows leave in 16-byte pieces (a lane holds one column of its tile: written
+        // directly that would be 64 two-byte stores per lane).  The tile buffers are free: the last unit's barrier
+        // came after every wavefront's last read of them.  Each wavefront uses its own 2 * 32 * RB bytes.
+        unsigned char* stage = smem + kbw * (2 * 32 * RB);
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = 8 * (r >> 2) + 4 * h + (r & 3);
-                dkp[row * rs + 32 * db] = bf16_bits(dkacc[db][r]);
-                dvp[row * rs + 32 * db] = bf16_bits(dvacc[db][r]);
+                *reinterpret_cast<uint16_t*>(stage + row * RB + (32 * db + n) * 2) = bf16_bits(dkacc[db][r]);
+                *reinterpret_cast<uint16_t*>(stage + 32 * RB + row * RB + (32 * db + n) * 2) = bf16_bits(dvacc[db][r]);
             }
-    }
-}
-
-// Indexed form of the two-wavefront kernel as a stream: instead of one short-lived workgroup per segment (whose
-// start-up -- table look-ups, K/V rows, first tile, all dependent memory round trips -- and scattered final stores
-// took a third of the kernel's time), a workgroup walks a share of its (sequence, kv head) pair's stream of steps,
-//     [K/V tile of segment s] [unit] [unit] ... [K/V tile of segment s+1] [unit] ...
-// through ONE software pipeline: tile copies run two steps ahead whatever the step is, a segment's K/V tile arrives
-// through the same double buffer as the Q / dO tiles (its rows are read back as the stationary operands), and the
-// finished dK / dV tile is stored while the next segment's first products run.
-template <int D>
-__global__ void __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2)))
-gca_bwd_dkdv_stream_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
-                           const uint16_t* __restrict__ v, const void* __restrict__ w, int w_is_bf16,
-                           const uint16_t* __restrict__ dout, const float* __restrict__ lse,
-                           const float* __restrict__ delta, void* __restrict__ dk_out, void* __restrict__ dv_out,
-                           ListWs ws, int W, int seg_max) {
-    constexpr int NT = 128;
-    constexpr int KS = D / 16, DB = D / 32;
-    constexpr int RB = D * 2, TILE = 64 * RB, BUF = 2 * TILE;   // Q tile then dO tile, or K tile then V tile
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * BUF];
-    __shared__ __attribute__((aligned(256))) float s_lse[2][2][64];
-    __shared__ __attribute__((aligned(256))) float s_dl[2][2][64];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, kbw = tid >> 6;     // kbw: which 32 key rows this wavefront owns
-    const int n = lane & 31, h = lane >> 5;
-
-    // ---- which share of which pair's stream.  Workgroup b runs on XCD b % 8: a pair's shares stay on one XCD,
-    //      so the Q / dO tiles its chunks keep re-reading stay in one L2.
-    const int64_t bidx = blockIdx.x / NUM_XCD;
-    const int64_t pair = (bidx / W) * NUM_XCD + blockIdx.x % NUM_XCD;
-    if (pair >= p.N * p.Hkv) return;
-    const int wi = (int)(bidx % W);
-    const int64_t nseq = pair / p.Hkv;
-    const int hk = (int)(pair % p.Hkv);
-    // (table values are clamped to their valid ranges wherever they become addresses: tables that were never built
-    // then give wrong numbers, not wild accesses)
-    const int seg_cap = (int)min((int64_t)INT32_MAX, p.N * p.C + (p.Z * p.K + seg_max - 1) / seg_max);
-    const int s_first = max(0, load_uniform_int(ws.wg_seg + nseq * (W + 1) + wi));
-    const int s_end = min(seg_cap, load_uniform_int(ws.wg_seg + nseq * (W + 1) + wi + 1));
-    if (s_first >= s_end) return;
-    const int ref_cap = (int)(p.Z * p.K - 1);
-    const int z_cap = (int)((nseq + 1) * p.zpn - 1);
-    const int64_t nc_cap = p.N * p.C - 1;
-    const int slot_cap = (int)min((int64_t)INT32_MAX, 2 * ((p.Z * p.K + seg_max - 1) / seg_max));
-    const int64_t rs = (int64_t)p.Hkv * D;          // row stride of the cache
-
-    const float c = p.sm_scale * LOG2E;
-    bf16x8 kB[KS], vB[KS];
-    bf16x8 onesB = {0, 0, 0, 0, 0, 0, 0, 0};
-    onesB[0] = (__bf16)1.0f;
-    onesB[1] = (__bf16)1.0f;
-    f32x16 dkacc[DB], dvacc[DB];
-
-    const TileLoader<D, NT> loader(tid, (int)p.q_rs);       // Q / dO tiles
-    const TileLoader<D, NT> loader_kv(tid, (int)rs);        // K / V tiles of a cache chunk
-    const int nqt = p.Q_CTX / 64;
-
-    // ---- the walk over the stream, two steps ahead of the math.  Everything here is wavefront-uniform.
-    struct Cursor {
-        int seg, len, cc, list0;   // current segment: its references, chunk, first position in refs
-        int t;                     // 0: the K/V tile step; 1 + (r * G + g) * nqt + qi: unit steps
-        int r, g, qi;              // reference, head of the group, query tile of the current unit step
-        int z, j;                  // (z, j) of reference list0 + r, requested one step early
-        bool valid;
-    } cur;
-    auto enter_segment = [&]() {
-        cur.valid = false;
-        while (cur.seg < s_end) {
-            cur.len = min(seg_max, load_uniform_int(ws.seg_len + cur.seg));
-            if (cur.len > 0) {
-                cur.cc = (int)min(nc_cap, (int64_t)max(0, load_uniform_int(ws.seg_chunk + cur.seg)));
-                cur.list0 = min(ref_cap + 1 - cur.len, max(0, load_uniform_int(ws.seg_start + cur.seg)));
-                cur.z = min(z_cap, max(0, load_uniform_int(ws.ref_zj + 2 * (int64_t)cur.list0)));
-                cur.j = min(p.K - 1, max(0, load_uniform_int(ws.ref_zj + 2 * (int64_t)cur.list0 + 1)));
-                cur.t = 0; cur.r = 0; cur.g = 0; cur.qi = 0;
-                cur.valid = true;
-                return;
-            }
-            ++cur.seg;
-        }
-    };
-    auto advance = [&]() {
-        if (cur.t > 0) {
-            if (++cur.qi == nqt) { cur.qi = 0; if (++cur.g == p.G) { cur.g = 0; ++cur.r; } }
-            if (cur.r == cur.len) { ++cur.seg; enter_segment(); return; }
-            if (cur.g == 0 && cur.qi == 0) {
-                cur.z = min(z_cap, max(0, load_uniform_int(ws.ref_zj + 2 * (int64_t)(cur.list0 + cur.r))));
-                cur.j = min(p.K - 1, max(0, load_uniform_int(ws.ref_zj + 2 * (int64_t)(cur.list0 + cur.r) + 1)));
-            }
-        }
-        ++cur.t;
-    };
-    struct Step {
-        int kind;      // 0: end of the share, 1: K/V tile, 2: unit
-        int last;      // unit: the last one of its segment (the tile is written out after it)
-        int seg;       // K/V tile: the segment (chunk id and partial slot are read when it is consumed)
-        float w;       // unit: the weight of its reference
-    };
-    // describes the cursor's step, issues its copies into buffer `buf`, moves the cursor on
-    auto make_step = [&](int buf) -> Step {
-        Step st = {0, 0, 0, 0.f};
-        if (!cur.valid) return st;
-        unsigned char* nb = smem + buf * BUF;
-        if (cur.t == 0) {
-            st.kind = 1;
-            st.seg = cur.seg;
-            const int64_t off = (int64_t)cur.cc * p.K_CTX * rs + (int64_t)hk * D;
-            loader_kv.issue(k + off, nb);
-            loader_kv.issue(v + off, nb + TILE);
-        } else {
-            st.kind = 2;
-            const int64_t z = cur.z;
-            const int j = cur.j;
-            const int hq = hk * p.G + cur.g;
-            const int qrow0 = cur.qi * 64;
-            const int64_t qoff = q_base_n(p, nseq, z, hq) + qrow0 * (int)p.q_rs;
-            const int64_t loffq = ((z * p.Hq + hq) * (int64_t)p.K + j) * p.Q_CTX + qrow0;
-            loader.issue(q + qoff, nb);
-            loader.issue(dout + qoff, nb + TILE);
-            async_row64(lse + loffq, s_lse[kbw][buf], lane);
-            async_row64(delta + loffq, s_dl[kbw][buf], lane);
-            st.w = load_w(w, w_is_bf16, z * p.K + j);
-            st.last = (cur.r == cur.len - 1 && cur.g == p.G - 1 && cur.qi == nqt - 1) ? 1 : 0;
-        }
-        advance();
-        return st;
-    };
-
-    const TrLane tr(lane);
-    const int fsw = swz(n);
-
-    // ---- operand fetch helpers (LDS -> registers)
-    // rows 32*rt + n of both tiles of a buffer, dims 16*ks + 8*h .. +7: the A operands of S and dP for 32 query
-    // rows, or (K/V step) this wavefront's key rows
-    auto load_rows = [&](int buf, int rt, bf16x8 (&a0)[KS], bf16x8 (&a1)[KS]) {
-        const unsigned char* b0 = smem + buf * BUF;
-        const int rowoff = (32 * rt + n) * RB;
+        // (a wavefront's own LDS writes and reads stay in order)
+        constexpr int PPR = RB / 16;                 // 16-byte pieces per row
+        uint16_t* dkp = (uint16_t*)dk_out + out_off + (int64_t)(32 * kbw) * rs;
+        uint16_t* dvp = (uint16_t*)dv_out + out_off + (int64_t)(32 * kbw) * rs;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            const int po = rowoff + (((2 * ks + h) ^ fsw) << 4);
-            a0[ks] = lds_read_b128(b0 + po);
-            a1[ks] = lds_read_b128(b0 + TILE + po);
-        }
-    };
-    // transposed B operands of dV and dK for the 16-query reduction step t4 (DB dim blocks each)
-    auto load_cols = [&](int buf, int t4, bf16x8 (&bdo)[DB], bf16x8 (&bq)[DB]) {
-        const unsigned char* qbuf = smem + buf * BUF;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-            const int o0 = tr.off(t4, db, RB);
-            bdo[db] = lds_read_tr_pair(qbuf + TILE + o0, qbuf + TILE + o0 + 8 * RB);
-            bq[db] = lds_read_tr_pair(qbuf + o0, qbuf + o0 + 8 * RB);
-        }
-    };
-    auto bias_operand = [&](float x) -> bf16x8 {
-        const __bf16 hi = (__bf16)x;
-        const __bf16 lo = (__bf16)(x - (float)hi);
-        bf16x8 a = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (h == 0) { a[0] = hi; a[1] = lo; }
-        return a;
-    };
-
-    bf16x8 aq[KS], ad[KS];
-    float ls[2] = {0.f, 0.f}, dl[2] = {0.f, 0.f};
-    // first operands of a step whose tiles have landed in buffer `buf`
-    // (a K/V step reads this wavefront's key rows, a unit the first 32 query rows; the lse / delta values only mean
-    // something for a unit; after the last step the reads hit a stale buffer and are never used)
-    auto prefetch = [&](const Step& st, int buf) {
-        load_rows(buf, st.kind == 1 ? kbw : 0, aq, ad);
-        ls[0] = s_lse[kbw][buf][n]; ls[1] = s_lse[kbw][buf][32 + n];
-        dl[0] = s_dl[kbw][buf][n];  dl[1] = s_dl[kbw][buf][32 + n];
-    };
-
-    // ---- prologue: the first two steps are requested, the first one's operands fetched
-    cur.seg = s_first;
-    enter_segment();
-    Step st0 = make_step(0);
-    Step st1 = make_step(1);
-    Step st2 = {0, 0, 0, 0.f};
-    wait_async_tiles();
-    __syncthreads();
-    prefetch(st0, 0);
-
-    int64_t out_off = 0;
-    int slot = -1;
-    // hands the step's buffer back (every LDS read of it has landed), requests the step after next into it and
-    // fetches the next step's first operands
-    auto mid_point = [&](int buf) {
-        __builtin_amdgcn_s_waitcnt(0x0070);        // vmcnt(0): the next step's tiles have landed; lgkmcnt(0): reads done
-        __syncthreads();
-        prefetch(st1, buf ^ 1);
-        st2 = make_step(buf);
-    };
-
-    // A share is a run of segments; a segment is its K/V tile step followed by its unit steps.
-    int pos = 0;
-    while (st0.kind != 0) {
-        {
-            const int buf = pos & 1;
-            // ---- K/V tile step: this wavefront's rows become the stationary operands K' and V'
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    kB[ks][e] = (__bf16)((float)aq[ks][e] * c);
-                    vB[ks][e] = (__bf16)((float)ad[ks][e] * p.sm_scale);
-                }
-#pragma unroll
-            for (int db = 0; db < DB; ++db)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
-            const int cc = (int)min(nc_cap, (int64_t)max(0, load_uniform_int(ws.seg_chunk + st0.seg)));
-            slot = min(slot_cap, load_uniform_int(ws.seg_slot + st0.seg));
-            out_off = (int64_t)cc * p.K_CTX * rs + (int64_t)hk * D;
-            mid_point(buf);
-        }
-        st0 = st1; st1 = st2; ++pos;
-        while (st0.kind == 2) {
-            const int buf = pos & 1;
-            // |w| rides in the bias (log2 |w| - lse), the sign of w goes on the rounded operands; weight 0 -> P~ = 0
-            const float aw = fabsf(st0.w);
-            const float lw = aw > 0.f ? __builtin_amdgcn_logf(aw) : -1e30f;
-            const bool wneg = st0.w < 0.f;
-            bf16x8 pA[2], dsA[2];
-            bf16x8 bdo[2][DB], bq[2][DB];
-#pragma unroll
-            for (int qt = 0; qt < 2; ++qt) {
-                // ---- S'' and dP'' for 32 query rows: queries in registers, key n in the lane
-                const bf16x8 bs = bias_operand(lw - ls[qt]);
-                const bf16x8 bd = bias_operand(-p.sm_scale * dl[qt]);
-                f32x16 s, dp;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aq[ks], kB[ks], s, 0, 0, 0);
-                    dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ad[ks], vB[ks], dp, 0, 0, 0);
-                }
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bs, onesB, s, 0, 0, 0);
-                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bd, onesB, dp, 0, 0, 0);
-                // fetch the transposed operands of the first 16 queries of this half while the products run
-                load_cols(buf, 2 * qt, bdo[0], bq[0]);
-                __builtin_amdgcn_sched_barrier(0);
-                // ---- element loop: registers 0..15 are queries 32*qt + 8*(r/4) + 4*h + r%4
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float pw = __builtin_amdgcn_exp2f(s[r]);
-                    pA[r >> 3][r & 7] = (__bf16)pw;
-                    dsA[r >> 3][r & 7] = (__bf16)(pw * dp[r]);
-                }
-                if (wneg) {
-#pragma unroll
-                    for (int t2 = 0; t2 < 2; ++t2) { pA[t2] = negate_bf16x8(pA[t2]); dsA[t2] = negate_bf16x8(dsA[t2]); }
-                }
-                // s and dp are dead now: their registers take the operands of the other 16 queries and the row
-                // operands of the next half (or, through mid_point, of the next step); they arrive under the products
-                load_cols(buf, 2 * qt + 1, bdo[1], bq[1]);
-                if (qt == 0) {
-                    load_rows(buf, 1, aq, ad);
-                    __builtin_amdgcn_sched_barrier(0);
-                } else {
-                    mid_point(buf);
-                }
-                // ---- dV += P~^T dO, dK += dS^T Q over these 32 queries (two 16-query reduction steps)
-#pragma unroll
-                for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-                    for (int db = 0; db < DB; ++db) {
-                        dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pA[t2], bdo[t2][db], dvacc[db], 0, 0, 0);
-                        dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsA[t2], bq[t2][db], dkacc[db], 0, 0, 0);
-                    }
-            }
-            if (st0.last) {
-                // ---- write the tile: register r of block db is key row 32*kbw + 8*(r/4) + 4*h + r%4, column 32*db + n
-                if (slot >= 0) {
-                    // (addresses are formed here, from an opaque copy of the slot, so that they are not kept in
-                    // registers from the moment the slot is known)
-                    int slot_here = slot;
-                    asm volatile("" : "+s"(slot_here));
-                    float* part = ws.partials + ((int64_t)slot_here * p.Hkv + hk) * 2 * (64 * D) + (32 * kbw + 4 * h) * D + n;
-                    float* part_v = part + 64 * D;
-#pragma unroll
-                    for (int db = 0; db < DB; ++db)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            const int row = 8 * (r >> 2) + (r & 3);          // + 4*h: in the base pointers
-                            part[row * D + 32 * db] = dkacc[db][r];
-                            part_v[row * D + 32 * db] = dvacc[db][r];
-                        }
-                } else {
-                    // (the row stride goes through an opaque copy so that the 32 row offsets are formed here, once
-                    // per segment, instead of being kept in registers across the whole walk)
-                    int rs_here = (int)rs;
-                    asm volatile("" : "+s"(rs_here));
-                    uint16_t* dkp = (uint16_t*)dk_out + out_off + (int64_t)(32 * kbw + 4 * h) * rs_here + n;
-                    uint16_t* dvp = (uint16_t*)dv_out + out_off + (int64_t)(32 * kbw + 4 * h) * rs_here + n;
-#pragma unroll
-                    for (int db = 0; db < DB; ++db)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            const int row = 8 * (r >> 2) + (r & 3);          // + 4*h: in the base pointers
-                            dkp[row * rs_here + 32 * db] = bf16_bits(dkacc[db][r]);
-                            dvp[row * rs_here + 32 * db] = bf16_bits(dvacc[db][r]);
-                        }
-                }
-            }
-            st0 = st1; st1 = st2; ++pos;
+        for (int i = 0; i < 32 * PPR / 64; ++i) {
+            const int piece = i * 64 + lane, row = piece / PPR, col8 = (piece % PPR) * 8;
+            const u32x4 a = *reinterpret_cast<const u32x4*>(stage + piece * 16);
+            const u32x4 b = *reinterpret_cast<const u32x4*>(stage + 32 * RB + piece * 16);
+            *reinterpret_cast<u32x4*>(dkp + (int64_t)row * rs + col8) = a;
+            *reinterpret_cast<u32x4*>(dvp + (int64_t)row * rs + col8) = b;
         }
     }
 }
@@ -1035,28 +735,16 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
     }
 }
 
-// Chunks whose list was cut into several segments: add the float partial tiles in segment order.  With
-// ZERO_EMPTY it also writes the zero gradient of chunks nobody referenced (the stream kernel skips those).
+// Chunks whose list was cut into several segments: add the float partial tiles in segment order.
 // grid = NC * Hkv workgroups; those of single-segment chunks return at once.
-template <int D, bool ZERO_EMPTY>
+template <int D>
 __global__ void __launch_bounds__(256)
 gca_bwd_dkdv_reduce_kernel(Params p, int seg_max, uint16_t* __restrict__ dk_out, uint16_t* __restrict__ dv_out, ListWs ws) {
     const int64_t cc = blockIdx.x / p.Hkv;
     const int hk = blockIdx.x % p.Hkv;
-    const int cnt = ws.count[cc];
-    const int sg = (cnt + seg_max - 1) / seg_max;
+    const int sg = (ws.count[cc] + seg_max - 1) / seg_max;
     const int64_t rs = (int64_t)p.Hkv * D;
     const int64_t out_off = cc * p.K_CTX * rs + (int64_t)hk * D;
-    if (ZERO_EMPTY && cnt == 0) {
-        // 16 bytes per thread: a row of one head is D bf16 = D/8 pieces
-        for (int i = threadIdx.x; i < 64 * (D / 8); i += 256) {
-            const int64_t off = out_off + (int64_t)(i / (D / 8)) * rs + (i % (D / 8)) * 8;
-            const u32x4 zero = {0u, 0u, 0u, 0u};
-            *reinterpret_cast<u32x4*>(dk_out + off) = zero;
-            *reinterpret_cast<u32x4*>(dv_out + off) = zero;
-        }
-        return;
-    }
     if (sg <= 1) return;
     const int slot0 = ws.slot_base[cc];
     for (int i = threadIdx.x; i < 64 * D; i += 256) {
@@ -1093,7 +781,7 @@ static int launch_dq_gs(const Params& p, const void* q, const void* k, const voi
 template <int D>
 static int launch_bwd_d(const Params& p, const void* q, const void* k, const void* v, const int64_t* idx, const void* w,
                         int wb, const void* dout, const float* lse, void* dq, void* dk, void* dv, float* dw,
-                        float* delta, hipStream_t s) {
+                        float* delta, void* lists, hipStream_t s) {
     int rc = GCA_OK;
     if (p.stages & GCA_STAGE_DQ) {
         if (p.G % 4 == 0) rc = launch_dq_gs<D, 4>(p, q, k, v, idx, w, wb, dout, lse, dq, delta, s);
@@ -1106,19 +794,10 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
     const int seg_per0 = 0;
     if (p.indexed) {
         // the list tables follow delta, the partial tiles follow the tables
-        const int upr = p.G * (p.Q_CTX / 64);
         char* tables = (char*)delta + delta_bytes(p);
-        ws = list_carve(p, SEG_MAX, upr, tables, tables + list_table_bytes(p, SEG_MAX, upr));
-        if ((p.stages & GCA_STAGE_LISTS) && (rc = list_build(p, SEG_MAX, upr, idx, ws, s)) != GCA_OK) return rc;
+        ws = list_carve(p, SEG_MAX, lists != nullptr ? lists : tables, tables + list_table_bytes(p, SEG_MAX));
+        if (lists == nullptr && (p.stages & GCA_STAGE_LISTS) && (rc = list_build(p, SEG_MAX, idx, ws, s)) != GCA_OK) return rc;
         if (!(p.stages & GCA_STAGE_DKDV)) {
-        } else if constexpr (D == 64 && USE_STREAM) {
-            // stream kernel: W shares per (sequence, kv head) pair, a pair's shares on one XCD
-            const int W = list_stream_wgs(p, SEG_MAX, upr);
-            const int64_t blocks = (p.N * p.Hkv + NUM_XCD - 1) / NUM_XCD * NUM_XCD * W;
-            if (blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
-            hipLaunchKernelGGL((gca_bwd_dkdv_stream_kernel<D>), dim3((unsigned)blocks), dim3(128), 0, s, p,
-                               (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
-                               delta, dk, dv, ws, W, SEG_MAX);
         } else {
             // segment slots per sequence: every chunk has one segment, plus one per SEG_MAX references
             const int seg_per = (int)(p.C + (p.zpn * p.K + SEG_MAX - 1) / SEG_MAX);
@@ -1135,7 +814,7 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
         }
         if (p.N * p.C * p.Hkv > 0x7fffffffLL) return GCA_ERR_SHAPE;
         if (p.stages & GCA_STAGE_REDUCE)
-            hipLaunchKernelGGL((gca_bwd_dkdv_reduce_kernel<D, D == 64 && USE_STREAM>), dim3((unsigned)(p.N * p.C * p.Hkv)), dim3(256), 0, s, p,
+            hipLaunchKernelGGL((gca_bwd_dkdv_reduce_kernel<D>), dim3((unsigned)(p.N * p.C * p.Hkv)), dim3(256), 0, s, p,
                                SEG_MAX, (uint16_t*)dk, (uint16_t*)dv, ws);
     } else {
         const int64_t blocks = p.Z * p.Hkv * p.K;
@@ -1157,18 +836,32 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
 size_t bwd_workspace_bytes(const gca_desc& d, bool indexed) {
     const Params p = make_params(d, indexed);
     size_t bytes = delta_bytes(p);
-    if (indexed) bytes += list_ws_bytes(p, SEG_MAX, p.G * (p.Q_CTX / 64));
+    if (indexed) bytes += list_ws_bytes(p, SEG_MAX);
     return bytes;
 }
 
 int launch_bwd_mfma(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v, const int64_t* indices,
                     const void* w, const void* dout, const float* lse, void* dq, void* dk, void* dv, float* dw,
-                    float* delta, hipStream_t s) {
+                    float* delta, void* lists, hipStream_t s) {
     if (!mfma_supported(d)) return GCA_ERR_UNSUPPORTED;
     const Params p = make_params(d, indexed);
     const int wb = d.w_dtype == GCA_BF16 ? 1 : 0;
-    if (d.D == 64) return launch_bwd_d<64>(p, q, k, v, indices, w, wb, dout, lse, dq, dk, dv, dw, delta, s);
-    return launch_bwd_d<128>(p, q, k, v, indices, w, wb, dout, lse, dq, dk, dv, dw, delta, s);
+    if (d.D == 64) return launch_bwd_d<64>(p, q, k, v, indices, w, wb, dout, lse, dq, dk, dv, dw, delta, lists, s);
+    return launch_bwd_d<128>(p, q, k, v, indices, w, wb, dout, lse, dq, dk, dv, dw, delta, lists, s);
+}
+
+// the generic kernels walk every chunk's list whole (one segment per chunk)
+constexpr int GENERIC_LIST_SEG_MAX = 1 << 30;
+
+size_t lists_table_bytes(const gca_desc& d, bool use_mfma) {
+    return list_table_bytes(make_params(d, true), use_mfma ? SEG_MAX : GENERIC_LIST_SEG_MAX);
+}
+
+int launch_lists_build(const gca_desc& d, bool use_mfma, const int64_t* indices, void* lists, hipStream_t s) {
+    const Params p = make_params(d, true);
+    const int seg_max = use_mfma ? SEG_MAX : GENERIC_LIST_SEG_MAX;
+    // no partial tiles are touched by the build
+    return list_build(p, seg_max, indices, list_carve(p, seg_max, lists, nullptr), s);
 }
 
 }  // namespace gca

@@ -124,9 +124,9 @@ int gca_bwd(const gca_desc* desc, const void* q, const void* k, const void* v, c
     if ((rc = pick_path(*desc, use_mfma, false)) != GCA_OK) return rc;
     if (use_mfma)
         return launch_bwd_mfma(*desc, false, q, k, v, nullptr, weights, dout, lse, dq, dk, dv, dw, (float*)workspace,
-                               (hipStream_t)stream);
+                               nullptr, (hipStream_t)stream);
     return launch_bwd_generic(*desc, false, q, k, v, nullptr, weights, dout, lse, dq, dk, dv, dw, (float*)workspace,
-                              (hipStream_t)stream);
+                              nullptr, (hipStream_t)stream);
 }
 
 int gca_fwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, const void* v_cache,
@@ -140,10 +140,10 @@ int gca_fwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, co
     return launch_fwd_generic(*desc, true, q, k_cache, v_cache, indices, weights, o, lse, (hipStream_t)stream);
 }
 
-int gca_bwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, const void* v_cache,
-                    const int64_t* indices, const void* weights, const void* dout, const float* lse,
-                    void* dq, void* dk_cache, void* dv_cache, float* dw,
-                    void* workspace, size_t workspace_bytes, void* stream) {
+int gca_bwd_indexed_lists(const gca_desc* desc, const void* q, const void* k_cache, const void* v_cache,
+                          const int64_t* indices, const void* weights, const void* dout, const float* lse,
+                          void* dq, void* dk_cache, void* dv_cache, float* dw,
+                          void* workspace, size_t workspace_bytes, const void* lists, size_t lists_bytes, void* stream) {
     int rc = check_desc(desc, true);
     if (rc != GCA_OK) return rc;
     if (!q || !k_cache || !v_cache || !indices || !weights || !dout || !lse || !dq || !dk_cache || !dv_cache || !dw)
@@ -151,11 +151,37 @@ int gca_bwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, co
     if (!workspace || workspace_bytes < gca_bwd_workspace_bytes(desc)) return GCA_ERR_WORKSPACE;
     bool use_mfma = false;
     if ((rc = pick_path(*desc, use_mfma, false)) != GCA_OK) return rc;
+    if (lists != nullptr && lists_bytes < lists_table_bytes(*desc, use_mfma)) return GCA_ERR_WORKSPACE;
     if (use_mfma)
         return launch_bwd_mfma(*desc, true, q, k_cache, v_cache, indices, weights, dout, lse, dq, dk_cache, dv_cache, dw,
-                               (float*)workspace, (hipStream_t)stream);
+                               (float*)workspace, const_cast<void*>(lists), (hipStream_t)stream);
     return launch_bwd_generic(*desc, true, q, k_cache, v_cache, indices, weights, dout, lse, dq, dk_cache, dv_cache, dw,
-                              (float*)workspace, (hipStream_t)stream);
+                              (float*)workspace, const_cast<void*>(lists), (hipStream_t)stream);
+}
+
+int gca_bwd_indexed(const gca_desc* desc, const void* q, const void* k_cache, const void* v_cache,
+                    const int64_t* indices, const void* weights, const void* dout, const float* lse,
+                    void* dq, void* dk_cache, void* dv_cache, float* dw,
+                    void* workspace, size_t workspace_bytes, void* stream) {
+    return gca_bwd_indexed_lists(desc, q, k_cache, v_cache, indices, weights, dout, lse, dq, dk_cache, dv_cache, dw,
+                                 workspace, workspace_bytes, nullptr, 0, stream);
+}
+
+size_t gca_lists_workspace_bytes(const gca_desc* desc) {
+    if (check_desc(desc, true) != GCA_OK) return 0;
+    bool use_mfma = false;
+    if (pick_path(*desc, use_mfma, false) != GCA_OK) return 0;
+    return lists_table_bytes(*desc, use_mfma);
+}
+
+int gca_lists_build(const gca_desc* desc, const int64_t* indices, void* lists, size_t lists_bytes, void* stream) {
+    int rc = check_desc(desc, true);
+    if (rc != GCA_OK) return rc;
+    if (!indices) return GCA_ERR_NULL;
+    bool use_mfma = false;
+    if ((rc = pick_path(*desc, use_mfma, false)) != GCA_OK) return rc;
+    if (!lists || lists_bytes < lists_table_bytes(*desc, use_mfma)) return GCA_ERR_WORKSPACE;
+    return launch_lists_build(*desc, use_mfma, indices, lists, (hipStream_t)stream);
 }
 
 int lmk_score(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, void* scores, void* stream) {

@@ -98,16 +98,21 @@ __device__ __forceinline__ const T* chunk_base(const Params& p, const T* base, c
 namespace gca {
 int launch_fwd_generic(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v,
                        const int64_t* indices, const void* w, void* o, float* lse, hipStream_t s);
+// `lists`: reference-list tables built earlier by launch_lists_build for the same descriptor and indices (the
+// LISTS stage is then skipped), or nullptr: the tables live in the workspace behind delta and are built by the call
 int launch_bwd_generic(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v,
                        const int64_t* indices, const void* w, const void* dout, const float* lse,
-                       void* dq, void* dk, void* dv, float* dw, float* delta, hipStream_t s);
+                       void* dq, void* dk, void* dv, float* dw, float* delta, void* lists, hipStream_t s);
 bool mfma_supported(const gca_desc& d);       // forward and backward
 bool mfma_fwd_supported(const gca_desc& d);   // forward only: any Q_CTX
 int launch_fwd_mfma(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v,
                     const int64_t* indices, const void* w, void* o, float* lse, hipStream_t s);
 int launch_bwd_mfma(const gca_desc& d, bool indexed, const void* q, const void* k, const void* v,
                     const int64_t* indices, const void* w, const void* dout, const float* lse,
-                    void* dq, void* dk, void* dv, float* dw, float* delta, hipStream_t s);
+                    void* dq, void* dk, void* dv, float* dw, float* delta, void* lists, hipStream_t s);
+// reference-list tables of the indexed backward for the kernel family `use_mfma` selects
+size_t lists_table_bytes(const gca_desc& d, bool use_mfma);
+int launch_lists_build(const gca_desc& d, bool use_mfma, const int64_t* indices, void* lists, hipStream_t s);
 int launch_lmk_score(const lmk_desc& d, const void* lq, const void* lk, void* scores, hipStream_t s);
 int launch_lmk_topk(const lmk_desc& d, const void* scores, const void* noise, int64_t* indices, float* weights,
                     void* ws, size_t ws_bytes, hipStream_t s);

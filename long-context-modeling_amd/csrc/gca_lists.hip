@@ -8,43 +8,20 @@ int64_t list_slot_bound(const Params& p, int seg_max) { return 2 * ((p.Z * p.K +
 
 static size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
-// Workgroups per (sequence, kv head) pair of the stream kernel: shares of about STREAM_TARGET steps, and never
-// smaller than two full segments so that shares stay balanced.  Depends on the shapes only.
-#ifndef STREAM_TARGET_VALUE
-#define STREAM_TARGET_VALUE 48
-#endif
-constexpr int STREAM_TARGET = STREAM_TARGET_VALUE;
-int list_stream_wgs(const Params& p, int seg_max, int upr) {
-    const int64_t refs = p.zpn * p.K;
-    const int64_t steps = refs * upr + p.C + (refs + seg_max - 1) / seg_max;     // upper bound per sequence
-    const int64_t seg_steps = 1 + (int64_t)seg_max * upr;
-#ifdef STREAM_NO_FLOOR
-    const int64_t tgt = STREAM_TARGET;
-#else
-    const int64_t tgt = STREAM_TARGET > 2 * seg_steps ? STREAM_TARGET : 2 * seg_steps;
-#endif
-    int64_t w = (steps + tgt - 1) / tgt;
-    if (w < 1) w = 1;
-    if (w > 8192) w = 8192;
-    return (int)w;
-}
-
-size_t list_table_bytes(const Params& p, int seg_max, int upr) {
-    const int64_t W = list_stream_wgs(p, seg_max, upr);
-    const size_t ints = (size_t)(5 * p.N * p.C + 4 + 3 * p.Z * p.K + 5 * list_seg_bound(p, seg_max) + 1 + p.N * (W + 1));
+size_t list_table_bytes(const Params& p, int seg_max) {
+    const size_t ints = (size_t)(5 * p.N * p.C + 4 + 3 * p.Z * p.K + 4 * list_seg_bound(p, seg_max));
     return align256(ints * sizeof(int));
 }
 
-size_t list_ws_bytes(const Params& p, int seg_max, int upr) {
+size_t list_ws_bytes(const Params& p, int seg_max) {
     const size_t tile = (size_t)p.K_CTX * p.D;
-    return list_table_bytes(p, seg_max, upr) + (size_t)list_slot_bound(p, seg_max) * p.Hkv * 2 * tile * sizeof(float);
+    return list_table_bytes(p, seg_max) + (size_t)list_slot_bound(p, seg_max) * p.Hkv * 2 * tile * sizeof(float);
 }
 
-ListWs list_carve(const Params& p, int seg_max, int upr, void* tables, void* partials) {
+ListWs list_carve(const Params& p, int seg_max, void* tables, void* partials) {
     ListWs ws;
     int* base = (int*)tables;
     const int64_t NC = p.N * p.C, sb = list_seg_bound(p, seg_max);
-    const int64_t W = list_stream_wgs(p, seg_max, upr);
     ws.count = base; base += NC;
     ws.start = base; base += NC;
     ws.seg_base = base; base += NC;
@@ -56,9 +33,7 @@ ListWs list_carve(const Params& p, int seg_max, int upr, void* tables, void* par
     ws.seg_chunk = base; base += sb;
     ws.seg_start = base; base += sb;
     ws.seg_len = base; base += sb;
-    ws.seg_slot = base; base += sb;
-    ws.seg_step = base; base += sb + 1;
-    ws.wg_seg = base; base += p.N * (W + 1);
+    ws.seg_slot = base;
     ws.partials = (float*)partials;
     return ws;
 }
@@ -90,11 +65,11 @@ gca_list_ref_kernel(Params p, const int64_t* __restrict__ indices, ListWs ws) {
     }
 }
 
-// One workgroup: exclusive scans of the reference counts, the segment counts, the slot counts and the stream
-// steps; writes each chunk's rows of the segment table and clears its scatter cursor.
+// One workgroup: exclusive scans of the reference counts, the segment counts and the slot counts; writes each
+// chunk's rows of the segment table and clears its scatter cursor.
 __global__ void __launch_bounds__(1024)
-gca_list_scan_kernel(Params p, int seg_max, int upr, ListWs ws) {
-    __shared__ int s_a[1024], s_b[1024], s_c[1024], s_d[1024];
+gca_list_scan_kernel(Params p, int seg_max, ListWs ws) {
+    __shared__ int s_a[1024], s_b[1024], s_c[1024];
     __shared__ int carry[4];
     const int tid = threadIdx.x;
     const int64_t NC = p.N * p.C;
@@ -105,23 +80,20 @@ gca_list_scan_kernel(Params p, int seg_max, int upr, ListWs ws) {
         const int cnt = cc < NC ? ws.count[cc] : 0;
         const int sg = cc < NC ? max(1, (cnt + seg_max - 1) / seg_max) : 0;
         const int sl = sg > 1 ? sg : 0;
-        const int st = cnt > 0 ? sg + cnt * upr : 0;          // one tile step per non-empty segment + its units
-        s_a[tid] = cnt; s_b[tid] = sg; s_c[tid] = sl; s_d[tid] = st;
+        s_a[tid] = cnt; s_b[tid] = sg; s_c[tid] = sl;
         __syncthreads();
         for (int off = 1; off < 1024; off <<= 1) {
             const int a = tid >= off ? s_a[tid - off] : 0;
             const int b = tid >= off ? s_b[tid - off] : 0;
             const int c3 = tid >= off ? s_c[tid - off] : 0;
-            const int d4 = tid >= off ? s_d[tid - off] : 0;
             __syncthreads();
-            s_a[tid] += a; s_b[tid] += b; s_c[tid] += c3; s_d[tid] += d4;
+            s_a[tid] += a; s_b[tid] += b; s_c[tid] += c3;
             __syncthreads();
         }
         if (cc < NC) {
             const int start = carry[0] + s_a[tid] - cnt;
             const int sb = carry[1] + s_b[tid] - sg;
             const int slot0 = carry[2] + s_c[tid] - sl;
-            const int step0 = carry[3] + s_d[tid] - st;
             ws.start[cc] = start;
             ws.seg_base[cc] = sb;
             ws.slot_base[cc] = slot0;
@@ -132,17 +104,13 @@ gca_list_scan_kernel(Params p, int seg_max, int upr, ListWs ws) {
                 ws.seg_start[sb + s] = start + s * seg_max;
                 ws.seg_len[sb + s] = len;
                 ws.seg_slot[sb + s] = sg > 1 ? slot0 + s : -1;
-                ws.seg_step[sb + s] = step0 + s * (1 + seg_max * upr);     // the segments before the last are full
             }
         }
         __syncthreads();
-        if (tid == 1023) { carry[0] += s_a[1023]; carry[1] += s_b[1023]; carry[2] += s_c[1023]; carry[3] += s_d[1023]; }
+        if (tid == 1023) { carry[0] += s_a[1023]; carry[1] += s_b[1023]; carry[2] += s_c[1023]; }
         __syncthreads();
     }
-    if (tid == 0) {
-        ws.nseg[0] = carry[1]; ws.nseg[1] = carry[2]; ws.nseg[2] = carry[3];
-        ws.seg_step[carry[1]] = carry[3];
-    }
+    if (tid == 0) { ws.nseg[0] = carry[1]; ws.nseg[1] = carry[2]; }
 }
 
 // Ascending sort of a[0, n) by all threads of the workgroup: bitonic network in the form whose compare-exchanges
@@ -193,38 +161,16 @@ gca_list_sort_kernel(Params p, ListWs ws) {
     }
 }
 
-// wg_seg[n][wi] = first segment of sequence n whose first step is at or after share wi of the sequence's stream
-__global__ void __launch_bounds__(256)
-gca_list_split_kernel(Params p, int W, ListWs ws) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= p.N * (W + 1)) return;
-    const int64_t n = i / (W + 1);
-    const int wi = (int)(i % (W + 1));
-    const int seg_lo = ws.seg_base[n * p.C];
-    const int seg_hi = n + 1 < p.N ? ws.seg_base[(n + 1) * p.C] : ws.nseg[0];
-    const int lo_step = ws.seg_step[seg_lo], total = ws.seg_step[seg_hi] - lo_step;
-    const int tgt = max(1, (total + W - 1) / W);
-    const int64_t want = (int64_t)lo_step + (int64_t)wi * tgt;
-    int a = seg_lo, b = seg_hi;                 // lower bound of `want` in seg_step[seg_lo, seg_hi)
-    while (a < b) {
-        const int m = (a + b) >> 1;
-        if (ws.seg_step[m] < want) a = m + 1; else b = m;
-    }
-    ws.wg_seg[i] = wi == W ? seg_hi : a;
-}
-
-int list_build(const Params& p, int seg_max, int upr, const int64_t* indices, const ListWs& ws, hipStream_t s) {
+int list_build(const Params& p, int seg_max, const int64_t* indices, const ListWs& ws, hipStream_t s) {
     const int64_t NC = p.N * p.C, R = p.Z * p.K;
-    // every table entry is a 32-bit int: reference ids, chunk ids, list positions, stream steps
-    if (NC > INT_MAX || R > INT_MAX || R * (int64_t)upr + list_seg_bound(p, seg_max) > INT_MAX) return GCA_ERR_SHAPE;
-    const int W = list_stream_wgs(p, seg_max, upr);
+    // every table entry is a 32-bit int: reference ids, chunk ids, list positions, segment numbers
+    if (NC > INT_MAX || R > INT_MAX || list_seg_bound(p, seg_max) > INT_MAX) return GCA_ERR_SHAPE;
     const unsigned rb = (unsigned)((R + 255) / 256);
     hipLaunchKernelGGL(gca_list_zero_kernel, dim3((unsigned)((NC + 255) / 256)), dim3(256), 0, s, NC, ws.count);
     hipLaunchKernelGGL((gca_list_ref_kernel<false>), dim3(rb), dim3(256), 0, s, p, indices, ws);
-    hipLaunchKernelGGL(gca_list_scan_kernel, dim3(1), dim3(1024), 0, s, p, seg_max, upr, ws);
+    hipLaunchKernelGGL(gca_list_scan_kernel, dim3(1), dim3(1024), 0, s, p, seg_max, ws);
     hipLaunchKernelGGL((gca_list_ref_kernel<true>), dim3(rb), dim3(256), 0, s, p, indices, ws);
     hipLaunchKernelGGL(gca_list_sort_kernel, dim3((unsigned)NC), dim3(256), 0, s, p, ws);
-    hipLaunchKernelGGL(gca_list_split_kernel, dim3((unsigned)((p.N * (W + 1) + 255) / 256)), dim3(256), 0, s, p, W, ws);
     return hipGetLastError() == hipSuccess ? GCA_OK : GCA_ERR_LAUNCH;
 }
 

@@ -874,7 +874,7 @@ constexpr int LMK_SEG_MAX = 1 << 30;       // every list is walked whole
 size_t lmk_bwd_ws_bytes(const lmk_desc& d) {
     const int kk = (int)((int64_t)d.topk < d.E ? d.topk : d.E);
     const size_t dsb = ((size_t)d.N * d.C * kk * sizeof(float) + 255) / 256 * 256;
-    return dsb + list_ws_bytes(lists_params(d, kk), LMK_SEG_MAX, 1);
+    return dsb + list_ws_bytes(lists_params(d, kk), LMK_SEG_MAX);
 }
 
 template <typename T>
@@ -886,11 +886,11 @@ static int launch_lmk_bwd_t(const lmk_desc& d, int kk, const void* lq, const voi
     const size_t dsb = ((size_t)R * kk * sizeof(float) + 255) / 256 * 256;
     const Params p = lists_params(d, kk);
     char* tables = (char*)wsp + dsb;
-    const ListWs ws = list_carve(p, LMK_SEG_MAX, 1, tables, tables + list_table_bytes(p, LMK_SEG_MAX, 1));
+    const ListWs ws = list_carve(p, LMK_SEG_MAX, tables, tables + list_table_bytes(p, LMK_SEG_MAX));
     hipLaunchKernelGGL(lmk_bwd_ds_kernel, dim3((unsigned)((R + 63) / 64)), dim3(64), 0, s, d, kk, w, dw, ds);
     hipLaunchKernelGGL((lmk_bwd_dq_kernel<T>), dim3((unsigned)R), dim3(256), 0, s, d, kk, (const T*)lk, idx, ds, (T*)dlq);
     if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
-    const int rc = list_build(p, LMK_SEG_MAX, 1, idx, ws, s);
+    const int rc = list_build(p, LMK_SEG_MAX, idx, ws, s);
     if (rc != GCA_OK) return rc;
     hipLaunchKernelGGL((lmk_bwd_dk_kernel<T>), dim3((unsigned)(d.N * d.E)), dim3(256), 0, s, d, kk, (const T*)lq, ds, (T*)dlk, ws);
     return hipGetLastError() == hipSuccess ? GCA_OK : GCA_ERR_LAUNCH;

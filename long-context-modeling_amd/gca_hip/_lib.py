@@ -22,6 +22,7 @@ SYMBOLS = (
     "gca_version", "gca_strerror", "gca_fwd", "gca_bwd_workspace_bytes", "gca_bwd", "gca_fwd_indexed",
     "gca_bwd_indexed", "lmk_score", "lmk_topk_workspace_bytes", "lmk_topk", "lmk_score_topk",
     "lmk_weights_bwd_workspace_bytes", "lmk_weights_bwd", "chunk_cache_append", "lmk_score_topk_static",
+    "gca_lists_workspace_bytes", "gca_lists_build", "gca_bwd_indexed_lists",
 )
 LMK_STATIC_SCRATCH_BYTES = 8 << 20
 GCA_ERR_SCRATCH_LIMIT = 7
@@ -78,6 +79,12 @@ def _declare(lib):
     lib.gca_fwd_indexed.argtypes = [D, P, P, P, I64P, P, P, FP, P]
     lib.gca_bwd_indexed.restype = ctypes.c_int
     lib.gca_bwd_indexed.argtypes = [D, P, P, P, I64P, P, P, FP, P, FP, FP, FP, P, ctypes.c_size_t, P]
+    lib.gca_lists_workspace_bytes.restype = ctypes.c_size_t
+    lib.gca_lists_workspace_bytes.argtypes = [D]
+    lib.gca_lists_build.restype = ctypes.c_int
+    lib.gca_lists_build.argtypes = [D, I64P, P, ctypes.c_size_t, P]
+    lib.gca_bwd_indexed_lists.restype = ctypes.c_int
+    lib.gca_bwd_indexed_lists.argtypes = [D, P, P, P, I64P, P, P, FP, P, FP, FP, FP, P, ctypes.c_size_t, P, ctypes.c_size_t, P]
     lib.lmk_score.restype = ctypes.c_int
     lib.lmk_score.argtypes = [L, P, P, P, P]
     lib.lmk_topk_workspace_bytes.restype = ctypes.c_size_t

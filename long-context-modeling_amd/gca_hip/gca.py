@@ -21,6 +21,7 @@ indices (Z, K) int64 with Z % N == 0.
 """
 from __future__ import annotations
 
+import collections
 import ctypes
 
 import torch
@@ -130,6 +131,73 @@ def gca_kv_cache(q, k, v, weights, sm_scale, sm_n=0.0):
 
 # ------------------------------------------------------------------------------- indexed form
 
+class _ListCache:
+    """Reference-list tables of the indexed backward, kept per retrieval.
+
+    The tables (which query chunks retrieved each cache chunk) depend on ``indices`` only, and the layers of a group
+    share one retrieval (model/DRT.py:816-824, :853-886), so the first backward that meets an ``indices`` tensor builds
+    them (``gca_lists_build``) and the other layers reuse them (``gca_bwd_indexed_lists``).  An entry is valid for the
+    same memory, version counter and descriptor shape; it keeps the tensor alive, so the memory cannot be handed to
+    another tensor while the entry exists.  ``enabled = False`` makes every backward build its own lists.
+    """
+    enabled = True
+
+    def __init__(self, capacity=8):
+        self._entries = collections.OrderedDict()
+        self._capacity = capacity
+
+    def tables(self, key_tensor, desc, idx):
+        dev = idx.device
+        sig = (desc.dtype, desc.Z, desc.K, desc.N, desc.C, desc.D, desc.Q_CTX, desc.K_CTX, desc.Hq, desc.Hkv, desc.path,
+               dev.index, tuple(key_tensor.shape))
+        key = (key_tensor.data_ptr(), key_tensor._version, sig)
+        stream = torch.cuda.current_stream(dev)
+        hit = self._entries.get(key)
+        if hit is not None:
+            self._entries.move_to_end(key)
+            _, tables, event, built_on = hit
+            if built_on != stream.cuda_stream:
+                stream.wait_event(event)
+            return tables
+        L = _lib.lib()
+        nbytes = L.gca_lists_workspace_bytes(ctypes.byref(desc))
+        tables = torch.empty(max(nbytes, 1), device=dev, dtype=torch.uint8)
+        rc = L.gca_lists_build(ctypes.byref(desc), _ptr(idx), _ptr(tables), nbytes, ctypes.c_void_p(stream.cuda_stream))
+        _lib.check(rc, "gca_lists_build")
+        event = torch.cuda.Event()
+        event.record(stream)
+        self._entries[key] = (key_tensor, tables, event, stream.cuda_stream)
+        while len(self._entries) > self._capacity:
+            self._entries.popitem(last=False)
+        return tables
+
+    def clear(self):
+        self._entries.clear()
+
+
+list_cache = _ListCache()
+
+
+def _bwd_indexed(desc, q, k_cache, v_cache, idx, weights, do, lse, dq, dkc, dvc, dw, key_tensor):
+    """gca_bwd_indexed with the lists taken from (or put into) the cache."""
+    L = _lib.lib()
+    dev = q.device
+    with torch.cuda.device(dev):
+        nbytes = L.gca_bwd_workspace_bytes(ctypes.byref(desc))
+        ws = torch.empty(nbytes // 4, device=dev, dtype=torch.float32)
+        # (under stream capture nothing runs yet: tables recorded there must not be served to a later eager call)
+        if _ListCache.enabled and not torch.cuda.is_current_stream_capturing():
+            tables = list_cache.tables(key_tensor, desc, idx)
+            rc = L.gca_bwd_indexed_lists(ctypes.byref(desc), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(idx), _ptr(weights),
+                                         _ptr(do), _ptr(lse), _ptr(dq), _ptr(dkc), _ptr(dvc), _ptr(dw), _ptr(ws), nbytes,
+                                         _ptr(tables), tables.numel(), _stream(dev))
+        else:
+            rc = L.gca_bwd_indexed(ctypes.byref(desc), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(idx), _ptr(weights),
+                                   _ptr(do), _ptr(lse), _ptr(dq), _ptr(dkc), _ptr(dvc), _ptr(dw), _ptr(ws), nbytes,
+                                   _stream(dev))
+    _lib.check(rc, "gca_bwd_indexed")
+
+
 def _check_indexed(q, k_cache, v_cache, indices, weights):
     assert q.is_cuda and q.is_contiguous() and q.dim() == 4
     assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape == v_cache.shape and k_cache.dim() == 4
@@ -171,14 +239,7 @@ class _AttentionIndexed(torch.autograd.Function):
         dkc, dvc = torch.empty_like(k_cache), torch.empty_like(v_cache)
         dw = torch.empty(weights.shape, device=q.device, dtype=torch.float32)
         desc = _desc(q, K, K_CTX, Hkv, weights, ctx.sm_scale, ctx.sm_n, N=N, C=C)
-        with torch.cuda.device(q.device):
-            L = _lib.lib()
-            nbytes = L.gca_bwd_workspace_bytes(ctypes.byref(desc))
-            ws = torch.empty(nbytes // 4, device=q.device, dtype=torch.float32)
-            rc = L.gca_bwd_indexed(ctypes.byref(desc), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(indices),
-                                   _ptr(weights), _ptr(do), _ptr(lse), _ptr(dq), _ptr(dkc), _ptr(dvc), _ptr(dw),
-                                   _ptr(ws), nbytes, _stream(q.device))
-        _lib.check(rc, "gca_bwd_indexed")
+        _bwd_indexed(desc, q, k_cache, v_cache, indices, weights, do, lse, dq, dkc, dvc, dw, indices)
         return dq, dkc, dvc, None, dw.to(ctx.w_dtype), None, None
 
 
@@ -229,6 +290,7 @@ class _AttentionTokens(torch.autograd.Function):
         if want_grad:
             ctx.save_for_backward(q_tok, k_cache, v_cache, idx, w, lse)
             ctx.args = (num_heads, float(sm_scale), float(sm_n), weights.dtype, weights.shape)
+            ctx.indices_src = indices          # the retrieval's own tensor: what the layers of a group share
         return o
 
     @staticmethod
@@ -246,14 +308,7 @@ class _AttentionTokens(torch.autograd.Function):
         dw = torch.zeros(w_shape, device=q_tok.device, dtype=torch.float32)      # last retrieval row: unused, gradient 0
         dwz = torch.empty((Z, kk), device=q_tok.device, dtype=torch.float32)
         desc = _desc(q_tok, kk, K_CTX, Dm // D, w, sm_scale, sm_n, N=Nc, C=Cc, token_shape=(Z, num_heads, S, D, 1))
-        with torch.cuda.device(q_tok.device):
-            L = _lib.lib()
-            nbytes = L.gca_bwd_workspace_bytes(ctypes.byref(desc))
-            ws = torch.empty(nbytes // 4, device=q_tok.device, dtype=torch.float32)
-            rc = L.gca_bwd_indexed(ctypes.byref(desc), _ptr(q_tok), _ptr(k_cache), _ptr(v_cache), _ptr(idx), _ptr(w),
-                                   _ptr(do), _ptr(lse), _ptr(dq), _ptr(dkc), _ptr(dvc), _ptr(dwz), _ptr(ws), nbytes,
-                                   _stream(q_tok.device))
-        _lib.check(rc, "gca_bwd_indexed")
+        _bwd_indexed(desc, q_tok, k_cache, v_cache, idx, w, do, lse, dq, dkc, dvc, dwz, ctx.indices_src)
         dw[:, :-1] = dwz.view(N, C - 1, kk)
         return dq, dkc, dvc, None, dw.to(w_dtype), None, None, None, None
 

@@ -176,3 +176,55 @@ def test_module_decode_matches_batch_form():
         for s0, n in ((0, 1), (1, 2), (62, 2)):
             step = mod.decode(hidden[:, C - 1, s0:s0 + n], m, 0)
             assert rel_err(step, full[:, C - 1, s0:s0 + n]) < 2e-2
+
+
+def test_lists_are_built_once_per_retrieval_and_reused_across_layers():
+    """Six layers sharing one retrieval (model/DRT.py:853-886): the first backward builds the reference lists, the
+    others reuse them; gradients are bit-identical to runs that build their own lists, and a changed ``indices``
+    tensor gets new lists."""
+    import gca_hip
+    from gca_hip import gca as G
+    N, C, S, Hq, Hkv, d, kk = 2, 9, 64, 4, 2, 64, 3
+    ck, cv = gen((N, C, S, Hkv * d), 201, 0.5, torch.bfloat16).cuda(), gen((N, C, S, Hkv * d), 202, 0.5, torch.bfloat16).cuda()
+    _, idx, w = orc.retrieve(gen((N, C, 32), 203), gen((N, C, 32), 204), kk)
+    idx, w = idx.cuda(), w.cuda()
+    qs = [gen((N, C, S, Hq * d), 210 + i, 0.5, torch.bfloat16).cuda() for i in range(6)]
+    dos = [gen((N, C, S, Hq * d), 220 + i, 1.0, torch.bfloat16).cuda() for i in range(6)]
+
+    def run():
+        outs = []
+        for q_tok, do in zip(qs, dos):
+            a = [t.detach().clone().requires_grad_() for t in (q_tok, ck, cv)]
+            o = gca_hip.attention_tokens(a[0], a[1], a[2], idx, w, Hq, sm_n=0.0)
+            o.backward(do)
+            outs.append([t.grad for t in a])
+        return outs
+
+    G.list_cache.clear()
+    G._ListCache.enabled = False
+    try:
+        ref = run()
+    finally:
+        G._ListCache.enabled = True
+    got = run()
+    assert len(G.list_cache._entries) == 1                       # one build served all six layers
+    for r, g in zip(ref, got):
+        for a, b in zip(r, g):
+            assert torch.equal(a, b)
+    # a different retrieval (same shape, new memory) is not served from the old lists
+    idx2 = idx.flip(-1).contiguous()
+    a = [t.detach().clone().requires_grad_() for t in (qs[0], ck, cv)]
+    gca_hip.attention_tokens(a[0], a[1], a[2], idx2, w, Hq, sm_n=0.0).backward(dos[0])
+    assert len(G.list_cache._entries) == 2
+    G._ListCache.enabled = False
+    try:
+        b = [t.detach().clone().requires_grad_() for t in (qs[0], ck, cv)]
+        gca_hip.attention_tokens(b[0], b[1], b[2], idx2, w, Hq, sm_n=0.0).backward(dos[0])
+    finally:
+        G._ListCache.enabled = True
+    for x, y in zip(a, b):
+        assert torch.equal(x.grad, y.grad)
+    # in-place change of the retrieval bumps its version: new lists
+    idx.add_(0)
+    gca_hip.attention_tokens(qs[0].clone().requires_grad_(), ck, cv, idx, w, Hq, sm_n=0.0).sum().backward()
+    assert len(G.list_cache._entries) == 3
