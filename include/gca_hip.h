@@ -104,7 +104,10 @@ typedef struct lmk_desc {
     int64_t C;              /* query landmarks (rows) per sequence */
     int64_t E;              /* candidate chunks per sequence */
     int32_t Dm;             /* landmark width */
-    int32_t causal;         /* 1: row c sees chunk e iff (E - C + c) > e, others are -inf */
+    int32_t causal;         /* 1: row c sees chunk e iff (E - C + c) > e, others are -inf.  This is
+                               _enc_dec_score_mask with max_chunk_win = -1 (model/DRT.py:590-607), the only value
+                               the reference's retrieval passes (:613, :840 call it with the default); the
+                               sliding-window variant (max_chunk_win >= 0) is not implemented */
     float hidden_size;      /* scores are divided by sqrt(hidden_size) */
     int32_t lmk_k_rows;     /* landmark rows allocated per sequence in lmk_k: sequence n starts at row
                                n * lmk_k_rows (a cache with spare capacity); 0 means E (dense).  Honoured by

@@ -37,6 +37,23 @@ namespace gca {
 // references per dkdv workgroup in the indexed form: longer lists are cut into segments of this many
 constexpr int SEG_MAX = 32;
 
+// Order of the indexed dk/dv workgroups.  All chunks of a (sequence, kv head) pair re-read the same Q / dO rows
+// (those of the pair's later query chunks), K times over.  P pairs are in flight at a time; workgroup b runs on XCD
+// b % 8, pair slot (b % 8) % P owns the 8 / P XCDs that share it and deals its segments to them in turn.  Measured
+// with uniformly random retrieval (B=8 H=12 d=64 L=16K k=8, and B=4 Hq=32 Hkv=8 d=128 L=32K k=16): P = 8, one pair
+// per XCD, is the fastest at d=64 (0.61 ms against 0.63 / 0.65 / 0.68 for P = 4 / 2 / 1) and all four are within
+// 3 % at d=128, where a pair's Q / dO rows (67 MB) exceed every L2 whatever the order.
+constexpr int dkdv_pairs_in_flight(int) { return 8; }
+template <int P>
+__device__ __forceinline__ void dkdv_pair_of_block(int64_t b, int seg_per, int64_t& pair, int64_t& segi) {
+    static_assert(NUM_XCD % P == 0, "pairs in flight must divide the XCD count");
+    const int x = (int)(b % NUM_XCD);
+    const int64_t lin = (b / NUM_XCD) * (NUM_XCD / P) + x / P;      // position in the slot's stream of segments
+    pair = (lin / seg_per) * P + x % P;
+    segi = lin % seg_per;
+}
+inline int64_t dkdv_grid(int64_t pairs, int seg_per, int P) { return (pairs + P - 1) / P * seg_per * P; }
+
 // ------------------------------------------------------------------------------------------- dq
 
 template <int D, int GS, bool INDEXED>
@@ -243,17 +260,15 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
     const uint16_t* vt;
     int64_t rs, out_off;     // key-row stride of the tile; element offset of the tile in the output
     if (INDEXED) {
-        // (sequence, kv head) pairs are dealt round-robin to the XCDs (workgroup b runs on XCD b % 8), so the
-        // Q / dO tiles a pair's chunks keep re-reading stay in one L2; seg_per = segment slots per sequence.
-        const int64_t idx = blockIdx.x / NUM_XCD;
-        const int64_t pair = (idx / seg_per) * NUM_XCD + blockIdx.x % NUM_XCD;
+        int64_t pair, segi;
+        dkdv_pair_of_block<dkdv_pairs_in_flight(D)>(blockIdx.x, seg_per, pair, segi);
         if (pair >= p.N * p.Hkv) return;
         const int64_t nseq = pair / p.Hkv;
         qseq = nseq;
         hk = (int)(pair % p.Hkv);
         const int seg_lo = ws.seg_base[nseq * p.C];
         const int seg_hi = nseq + 1 < p.N ? ws.seg_base[(nseq + 1) * p.C] : ws.nseg[0];
-        const int seg = seg_lo + (int)(idx % seg_per);
+        const int seg = seg_lo + (int)segi;
         if (seg >= seg_hi) return;
         const int64_t cc = ws.seg_chunk[seg];
         list0 = ws.seg_start[seg];
@@ -529,17 +544,15 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
     const uint16_t* vt;
     int64_t rs, out_off;     // key-row stride of the tile; element offset of the tile in the output
     if (INDEXED) {
-        // (sequence, kv head) pairs are dealt round-robin to the XCDs (workgroup b runs on XCD b % 8), so the
-        // Q / dO tiles a pair's chunks keep re-reading stay in one L2; seg_per = segment slots per sequence.
-        const int64_t idx = blockIdx.x / NUM_XCD;
-        const int64_t pair = (idx / seg_per) * NUM_XCD + blockIdx.x % NUM_XCD;
+        int64_t pair, segi;
+        dkdv_pair_of_block<dkdv_pairs_in_flight(D)>(blockIdx.x, seg_per, pair, segi);
         if (pair >= p.N * p.Hkv) return;
         const int64_t nseq = pair / p.Hkv;
         qseq = nseq;
         hk = (int)(pair % p.Hkv);
         const int seg_lo = ws.seg_base[nseq * p.C];
         const int seg_hi = nseq + 1 < p.N ? ws.seg_base[(nseq + 1) * p.C] : ws.nseg[0];
-        const int seg = seg_lo + (int)(idx % seg_per);
+        const int seg = seg_lo + (int)segi;
         if (seg >= seg_hi) return;
         const int64_t cc = ws.seg_chunk[seg];
         list0 = ws.seg_start[seg];
@@ -801,7 +814,7 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
         } else {
             // segment slots per sequence: every chunk has one segment, plus one per SEG_MAX references
             const int seg_per = (int)(p.C + (p.zpn * p.K + SEG_MAX - 1) / SEG_MAX);
-            const int64_t blocks = (p.N * p.Hkv + NUM_XCD - 1) / NUM_XCD * NUM_XCD * seg_per;
+            const int64_t blocks = xcd_grid(dkdv_grid(p.N * p.Hkv, seg_per, dkdv_pairs_in_flight(D)));
             if (blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
             if constexpr (D == 64)
                 hipLaunchKernelGGL((gca_bwd_dkdv2_mfma_kernel<D, true>), dim3((unsigned)blocks), dim3(128), 0, s, p,
