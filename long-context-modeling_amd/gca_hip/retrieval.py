@@ -73,17 +73,64 @@ def landmark_topk(scores, topk, causal=True, noise=None):
     return indices, weights
 
 
+FUSED_MIN_BYTES = 128 << 20
+
+
+def landmark_score_topk(lmk_q, lmk_k, topk, hidden_size=None, causal=True, noise=None, return_scores=True,
+                        fused=None):
+    """Scoring and selection through the one-call entry point ``lmk_score_topk`` (model/DRT.py:612-627).
+    Returns (scores or None, indices, weights).  With ``return_scores=False`` and a score matrix of at least
+    ``FUSED_MIN_BYTES`` the matrix is never written: the fused kernel (bf16, width a multiple of 64, at least 32
+    query rows, k <= 32) selects while it scores.  It is the slower of the two forms (the memory is what it saves),
+    so smaller requests and shapes it does not take go through ``landmark_scores`` + ``landmark_topk`` and drop the
+    scores afterwards.  ``fused=True`` / ``False`` overrides the size rule."""
+    assert lmk_q.is_cuda and lmk_q.dim() == 3 and lmk_k.dim() == 3 and lmk_q.dtype in _DT and lmk_k.dtype == lmk_q.dtype
+    lmk_q = lmk_q.contiguous()
+    lmk_k, rows = _dense_or_strided(lmk_k)
+    N, C, Dm = lmk_q.shape
+    E = lmk_k.shape[1]
+    assert lmk_k.shape[0] == N and lmk_k.shape[2] == Dm
+    hidden_size = Dm if hidden_size is None else hidden_size
+    kk = min(E, int(topk))
+    if noise is not None:
+        assert noise.shape == (N, C, E) and noise.dtype == lmk_q.dtype
+        noise = noise.contiguous()
+    dev = lmk_q.device
+    if fused is None:
+        fused = N * C * E * lmk_q.element_size() >= FUSED_MIN_BYTES
+    if return_scores or not fused:
+        scores = landmark_scores(lmk_q, lmk_k, hidden_size, causal)
+        indices, weights = landmark_topk(scores, topk, causal, noise)
+        return (scores if return_scores else None), indices, weights
+    indices = torch.empty((N, C, kk), device=dev, dtype=torch.int64)
+    weights = torch.empty((N, C, kk), device=dev, dtype=torch.float32)
+    desc = _lmk_desc(lmk_q.dtype, topk, N, C, E, Dm, causal, hidden_size, rows)
+    with torch.cuda.device(dev):
+        L = _lib.lib()
+        nbytes = L.lmk_topk_workspace_bytes(ctypes.byref(desc))
+        ws = torch.empty(max(nbytes // 8, 1), device=dev, dtype=torch.int64)
+        rc = L.lmk_score_topk(ctypes.byref(desc), _ptr(lmk_q), _ptr(lmk_k), _ptr(noise), None, _ptr(indices),
+                              _ptr(weights), _ptr(ws), nbytes, _stream(dev))
+    if rc == _lib.GCA_ERR_UNSUPPORTED:
+        full = landmark_scores(lmk_q, lmk_k, hidden_size, causal)
+        indices, weights = landmark_topk(full, topk, causal, noise)
+        return None, indices, weights
+    _lib.check(rc, "lmk_score_topk")
+    return None, indices, weights
+
+
 class _Retrieve(torch.autograd.Function):
     """Scoring + selection with a backward: the gradient of the weights flows to both landmark
     embeddings (what autograd does through model/DRT.py:612 and :626-627); the selection is constant."""
 
     @staticmethod
-    def forward(ctx, lmk_q, lmk_k, topk, hidden_size, causal, noise):
+    def forward(ctx, lmk_q, lmk_k, topk, hidden_size, causal, noise, return_scores):
         lmk_q, lmk_k = lmk_q.contiguous(), lmk_k.contiguous()
-        scores = landmark_scores(lmk_q, lmk_k, hidden_size, causal)
-        indices, weights = landmark_topk(scores, topk, causal, noise)
+        scores, indices, weights = landmark_score_topk(lmk_q, lmk_k, topk, hidden_size, causal, noise, return_scores)
         ctx.save_for_backward(lmk_q, lmk_k, indices, weights)
         ctx.hidden, ctx.topk, ctx.causal = float(hidden_size), int(topk), bool(causal)
+        if scores is None:
+            scores = lmk_q.new_empty(0)
         ctx.mark_non_differentiable(scores, indices)
         return scores, indices, weights
 
@@ -102,20 +149,20 @@ class _Retrieve(torch.autograd.Function):
             rc = L.lmk_weights_bwd(ctypes.byref(desc), _ptr(lmk_q), _ptr(lmk_k), _ptr(indices), _ptr(weights),
                                    _ptr(dweights), _ptr(dlq), _ptr(dlk), _ptr(ws), nbytes, _stream(lmk_q.device))
         _lib.check(rc, "lmk_weights_bwd")
-        return dlq, dlk, None, None, None, None
+        return dlq, dlk, None, None, None, None, None
 
 
-def landmark_retrieve(lmk_q, lmk_k, topk, hidden_size=None, causal=True, noise=None):
+def landmark_retrieve(lmk_q, lmk_k, topk, hidden_size=None, causal=True, noise=None, return_scores=True):
     """Scoring + selection in one call.  Returns (scores, indices, weights); ``weights`` carries the
-    gradient to ``lmk_q`` and ``lmk_k``."""
+    gradient to ``lmk_q`` and ``lmk_k``.  ``return_scores=False`` returns None for the scores and lets the fused
+    kernel skip the (N, C, E) matrix (see ``landmark_score_topk``)."""
     assert lmk_q.is_cuda and lmk_q.dim() == 3 and lmk_k.dim() == 3
     hidden_size = lmk_q.shape[-1] if hidden_size is None else hidden_size
     if not (torch.is_grad_enabled() and (lmk_q.requires_grad or lmk_k.requires_grad)):
         # inference: no copy of a landmark store that is a view with spare capacity
-        scores = landmark_scores(lmk_q, lmk_k, hidden_size, causal)
-        indices, weights = landmark_topk(scores, topk, causal, noise)
-        return scores, indices, weights
-    return _Retrieve.apply(lmk_q, lmk_k, topk, hidden_size, causal, noise)
+        return landmark_score_topk(lmk_q, lmk_k, topk, hidden_size, causal, noise, return_scores)
+    scores, indices, weights = _Retrieve.apply(lmk_q, lmk_k, topk, hidden_size, causal, noise, return_scores)
+    return (scores if return_scores else None), indices, weights
 
 
 def landmark_retrieve_static(lmk_q, lmk_k, topk, out_indices, out_weights, hidden_size=None, causal=True, noise=None):
@@ -165,7 +212,7 @@ def gca_layer(q_all, chunk_k, chunk_v, lmk_q, lmk_k, topk, sm_n=0.0, hidden_size
     Returns (out (N, C, Hq, S, d), indices (N, C, kk), weights (N, C, kk))."""
     from .gca import attention_indexed, gca_kv_cache_indexed
     N, C, Hq, S, d = q_all.shape
-    _, indices, weights = landmark_retrieve(lmk_q, lmk_k, topk, hidden_size, True, noise)
+    _, indices, weights = landmark_retrieve(lmk_q, lmk_k, topk, hidden_size, True, noise, return_scores=False)
     out = torch.zeros_like(q_all)
     if C > 1:
         kk = indices.shape[-1]
