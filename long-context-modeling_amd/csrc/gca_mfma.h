@@ -9,9 +9,10 @@
 // 16t + 8 + 4h + c, which is the order C registers 8*(t%2) .. +7 of 32-row tile t/2 come in.
 //
 // LDS tiles are 64 rows of D bf16 without padding; the 16-byte pieces of a row are XOR-swizzled
-// with swz(row) so that the three access patterns used here are all bank-conflict free:
-// 16-byte writes of a row's pieces, 16-byte operand reads of 8 consecutive rows at one piece, and
-// ds_read_tr16_b64 patches of 4 consecutive rows x 32 bytes.
+// with swz(row) so that the three access patterns used here spread over the banks: 16-byte writes of a
+// row's pieces, 16-byte operand reads of 8 consecutive rows at one piece, and ds_read_tr16_b64 patches of
+// 4 consecutive rows x 32 bytes.  Not conflict-free: the counters show 0.3-0.4 conflict cycles per
+// LDS-active cycle in the attention kernels (an unswizzled tile would collide 8 ways on the operand reads).
 #pragma once
 #include "gca_common.h"
 

@@ -85,8 +85,8 @@ def test_fused_not_causal():
 
 
 def test_size_rule_and_scores_on_request():
-    """``fused=None``: small score matrices take the two launches even without scores; with scores the call returns
-    the bits of ``landmark_scores``.  Either way the selection is the fused kernel's."""
+    """``fused=None``: score matrices below 2 GiB take the two launches even without scores; with scores the call
+    returns the bits of ``landmark_scores``.  Either way the selection is the fused kernel's."""
     import gca_hip
     lq, lk = _landmarks(1, 200, 2300, 128, 900)
     _, ref_idx, ref_w, idx_f, w_f = _both(lq, lk, 8, hidden=96.0)
