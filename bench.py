@@ -81,6 +81,19 @@ def measured_traffic(profile=None):
     return out
 
 
+def measured_simd_shares(profile=None):
+    """{kernel: (MFMA busy share, other VALU issue share)} of the dispatch's SIMD cycles, from the tracked counter
+    summary (lines "SIMD_TIME_SHARE <kernel> <mfma> <valu>")."""
+    path = os.path.join(ROOT, profile or TRAFFIC_PROFILE)
+    out = {}
+    if os.path.exists(path):
+        for line in open(path):
+            m = re.match(r"^SIMD_TIME_SHARE\s+(\w+)\s+([\d.]+)\s+([\d.]+)\s*$", line.strip())
+            if m:
+                out[m.group(1)] = (float(m.group(2)), float(m.group(3)))
+    return out
+
+
 # ----------------------------------------------------------------------------------------- config 2
 
 def cfg2_inputs(torch, dev, seed, N=8, C=256, H=12, S=64, d=64):
@@ -508,6 +521,13 @@ def main():
                 "kernel_ms": {k_: round(v, 4) for k_, v in kt.items()},
                 "per_kernel_frac": {k_: bound_of(per_kernel[k_]["flops"], per_kernel[k_]["bytes"], kt[k_] * 1e-3)["frac"]
                                     for k_ in per_kernel},
+                "simd_time_share": {"note": "matrix and vector instructions do not overlap on a SIMD of this GPU (measured: "
+                                            "two wavefronts, one issuing MFMA 32x32x16, one VALU, take the sum of their "
+                                            "times), so MFMA busy + VALU issue cycles is the ceiling that binds these "
+                                            "kernels; shares of the dispatch's SIMD cycles from the tracked counters",
+                                    "source": TRAFFIC_PROFILE,
+                                    **{k_: {"mfma": v[0], "valu": v[1], "busy": round(v[0] + v[1], 3)}
+                                       for k_, v in measured_simd_shares().items() if k_ in per_kernel}},
                 "step": bound_of(step_work["flops"], step_work["bytes"], dt),
                 "stream_model": {"note": "gather-stream bytes (every query chunk streams its K retrieved chunks); not a "
                                          "ceiling for the indexed kernels, whose re-reads hit the caches",
