@@ -379,6 +379,7 @@ constexpr int TOPK_TILE = 2048;      // keys per LDS tile (rows longer than TOPK
 constexpr int TOPK_SMALL = 256;      // tile for short rows: fewer sorting stages
 constexpr int TOPK_THREADS = 256;
 constexpr int TOPK_MAX_KP = 128;     // largest supported power-of-two k
+constexpr int TOPK_FILTER_CAP = 256;  // keys one tile may pass the threshold filter of lmk_topk_reg_kernel
 
 __device__ __forceinline__ uint32_t sortable_bits(float v) {
     if (v != v) return 0xffffffffu;                 // NaN ranks above everything, as in torch.topk
@@ -490,6 +491,18 @@ __device__ __forceinline__ void merge_from(KT (&a)[KP], const KT (&b)[KP]) {
                 a[l] = sw ? x : y;
             }
         }
+}
+
+// Inserts x into the descending list a (the smallest entry falls off); branch-free.
+template <typename KT, int KP>
+__device__ __forceinline__ void insert_desc(KT (&a)[KP], KT x) {
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+        const bool keep = a[i] > x;
+        const KT hi = keep ? a[i] : x;
+        x = keep ? x : a[i];
+        a[i] = hi;
+    }
 }
 
 // Every thread passes its KP sorted keys; on return thread 0 holds the KP largest of the workgroup,
@@ -661,26 +674,106 @@ lmk_topk_reg_kernel(lmk_desc d, int kk, int nseg, int64_t seg_len, int64_t row0,
     const int64_t scan_end = min(d.E, max(limit, (int64_t)kk));
     const int64_t lo = (int64_t)seg * seg_len;
     const int64_t hi = min(lo + seg_len, scan_end);
+    // The first tile goes through the tournament.  From then on thread 0 holds the segment's KP best keys so far and
+    // their smallest is a threshold every later key must beat: the few that do (about KP * tile / position of them
+    // per tile on unordered data) are collected in LDS and inserted by thread 0.  A tile that collects more than
+    // the list holds (data ascending along the row) falls back to the tournament, with the keys already in registers.
+    // (A cheaper first threshold -- the smallest of KP group maxima -- was tried: it lets through so many keys that
+    // thread 0's serial inserts cost more than the tournament for k >= 16 and for 64-bit keys.)
+    __shared__ KT s_tau;
+    __shared__ int s_cnt;
+    __shared__ KT s_cand[TOPK_FILTER_CAP];
+    constexpr int VN = Vec16<T>::N;
+    const T* srow = scores + row * d.E;
+    const T* nrow = noise != nullptr ? noise + row * d.E : nullptr;
+    const bool vec = KP >= VN && sizeof(KT) * KP <= 128 && d.E % VN == 0 && ((uintptr_t)scores % 16 == 0) &&
+                     ((uintptr_t)noise % 16 == 0);
     KT best[KP];
 #pragma unroll
     for (int i = 0; i < KP; ++i) best[i] = 0;
+    if (tid == 0) { s_tau = 0; s_cnt = 0; }
+    __syncthreads();
+    bool first = true;
     for (int64_t pos = lo; pos < hi || pos == lo; pos += (int64_t)TOPK_THREADS * KP) {
         KT a[KP];
+        if (vec) {
+            // 16-byte loads: vector v of this thread covers candidates pos + (v * TOPK_THREADS + tid) * VN .. + VN - 1
 #pragma unroll
-        for (int i = 0; i < KP; ++i) {
-            const int64_t e = pos + (int64_t)i * TOPK_THREADS + tid;       // coalesced across the workgroup
-            KT key = 0;
-            if (e < hi) {
-                float sv = to_f(scores[row * d.E + e]);
-                if (noise != nullptr) sv = round_like<T>(sv + to_f(noise[row * d.E + e]));
-                if (d.causal && !(e < limit)) sv = -INFINITY;
-                key = SegKey<T>::make(sv, e, lo);
+            for (int v = 0; v < (KP >= VN ? KP / VN : 1); ++v) {
+                const int64_t e0 = pos + ((int64_t)v * TOPK_THREADS + tid) * VN;
+                union { uint4 u; T t[VN]; } sc, nz;
+                sc.u = make_uint4(0, 0, 0, 0);
+                nz.u = sc.u;
+                if (e0 < hi) {                    // e0 + VN <= E: e0 and E are multiples of VN
+                    sc.u = *reinterpret_cast<const uint4*>(srow + e0);
+                    if (noise != nullptr) nz.u = *reinterpret_cast<const uint4*>(nrow + e0);
+                }
+#pragma unroll
+                for (int j = 0; j < VN; ++j) {
+                    const int64_t e = e0 + j;
+                    KT key = 0;
+                    if (e < hi) {
+                        float sv = to_f(sc.t[j]);
+                        if (noise != nullptr) sv = round_like<T>(sv + to_f(nz.t[j]));
+                        if (d.causal && !(e < limit)) sv = -INFINITY;
+                        key = SegKey<T>::make(sv, e, lo);
+                    }
+                    if (v * VN + j < KP) a[v * VN + j] = key;
+                }
             }
-            a[i] = key;
+        } else {
+#pragma unroll
+            for (int i = 0; i < KP; ++i) {
+                const int64_t e = pos + (int64_t)i * TOPK_THREADS + tid;       // coalesced across the workgroup
+                KT key = 0;
+                if (e < hi) {
+                    float sv = to_f(srow[e]);
+                    if (noise != nullptr) sv = round_like<T>(sv + to_f(nrow[e]));
+                    if (d.causal && !(e < limit)) sv = -INFINITY;
+                    key = SegKey<T>::make(sv, e, lo);
+                }
+                a[i] = key;
+            }
         }
-        sort_desc_regs<KT, KP>(a);
-        block_tournament<KT, KP>(a, xch, tid);
-        if (tid == 0) merge_from<KT, KP>(best, a);
+        // 64-bit keys with KP = 32 fill the register file as it is: that variant keeps the plain tournament
+        constexpr bool FILTER = sizeof(KT) * KP <= 128;
+        bool tournament = first || !FILTER;  // the first tile has no threshold yet
+        if (FILTER && !first) {
+            const KT tau = s_tau;
+            bool any = false;
+#pragma unroll
+            for (int i = 0; i < KP; ++i) any |= a[i] > tau;
+            if (any) {
+#pragma unroll
+                for (int i = 0; i < KP; ++i)
+                    if (a[i] > tau) {
+                        const int slot = atomicAdd(&s_cnt, 1);
+                        if (slot < TOPK_FILTER_CAP) s_cand[slot] = a[i];
+                    }
+            }
+            __syncthreads();
+            const int n = s_cnt;                 // thread 0 clears it only when n <= CAP: late readers still see "no fallback"
+            tournament = n > TOPK_FILTER_CAP;
+            if (!tournament) {
+                if (tid == 0) {
+                    for (int i = 0; i < n; ++i) insert_desc<KT, KP>(best, s_cand[i]);
+                    s_tau = best[KP - 1];
+                    s_cnt = 0;
+                }
+                __syncthreads();
+            }
+        }
+        if (tournament) {
+            sort_desc_regs<KT, KP>(a);
+            block_tournament<KT, KP>(a, xch, tid);
+            if (tid == 0) {
+                merge_from<KT, KP>(best, a);
+                s_tau = best[KP - 1];
+                s_cnt = 0;
+            }
+            __syncthreads();
+        }
+        first = false;
     }
     if (tid == 0)
 #pragma unroll
@@ -862,17 +955,6 @@ __device__ __forceinline__ uint64_t fused_global_key(uint32_t k, int64_t lo) {
 }
 __device__ __forceinline__ uint64_t fused_global_key(uint64_t k, int64_t lo) {
     return k == 0 ? 0 : fused_global_key((uint32_t)(k >> 32), (uint32_t)k, lo);
-}
-
-template <typename KT, int KP>
-__device__ __forceinline__ void insert_desc(KT (&a)[KP], KT x) {
-#pragma unroll
-    for (int i = 0; i < KP; ++i) {
-        const bool keep = a[i] > x;
-        const KT hi = keep ? a[i] : x;
-        x = keep ? x : a[i];
-        a[i] = hi;
-    }
 }
 
 // indices / weights of one row from its kk best global keys (sorted); same arithmetic as emit_row
