@@ -71,6 +71,30 @@ def test_topk_gumbel_noise_selects_but_does_not_weigh(dtype):
     assert not torch.equal(idx_ref, _topk_ref(scores, k)[0])
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("k", [1, 8, 16, 32])
+@pytest.mark.parametrize("shape", ["random", "ascending", "descending", "constant", "sawtooth"])
+def test_topk_rows_longer_than_a_tile(shape, k, dtype):
+    """Rows of several tiles: after the first tile the kernel only looks at keys above the running k-th best.
+    Ascending rows pass every key (the candidate list overflows and the tile falls back to the tournament),
+    descending and constant rows pass none, a sawtooth alternates; E = 9001 is odd, so these rows also take the
+    scalar loads, E = 9000 the 16-byte ones; with noise both tensors are read that way."""
+    import gca_hip
+    for E in (9000, 9001):
+        C = 3
+        g = torch.Generator().manual_seed(40 + k)
+        base = torch.arange(E, dtype=torch.float32)
+        row = {"random": torch.randn(E, generator=g), "ascending": base / 64, "descending": -base / 64,
+               "constant": torch.full((E,), 0.5), "sawtooth": (base % 257) / 16}[shape]
+        scores = torch.stack([row, row.flip(0), torch.randn(E, generator=g)]).view(1, C, E).to(dtype)
+        noise = (torch.randn(1, C, E, generator=g) * 0.25).to(dtype)
+        for nz in (None, noise):
+            idx_ref, w_ref = _topk_ref(scores, k, False, nz)
+            idx, w = gca_hip.landmark_topk(scores.cuda(), k, causal=False, noise=None if nz is None else nz.cuda())
+            assert torch.equal(idx.cpu(), idx_ref), (shape, k, E, nz is not None)
+            assert (w.cpu() - w_ref).abs().max() <= 1e-6
+
+
 def test_topk_long_row_uses_segments():
     # one row long enough to be cut into segments and merged (decode at extreme context)
     import gca_hip
