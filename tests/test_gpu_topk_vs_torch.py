@@ -5,7 +5,7 @@
     slot for slot -- there is nothing to break ties on;
   * rows with exact ties (ordinary bf16 scores): the selected VALUES are the same multiset in the same order, and
     every index the two disagree on sits at a tied value.  How the library orders ties is recorded (printed and
-    written to gpurun_out/topk_ties.txt when that folder exists), not asserted: the kernels use the canonical rule
+    written to $GCA_TEST_RECORD_DIR/topk_ties.txt when that variable names a folder), not asserted: the kernels use the canonical rule
     "higher value first, then lower index".
 """
 import os
@@ -80,6 +80,7 @@ def test_tied_bf16_rows_values_agree_and_tie_order_is_recorded():
             f"{int(differ.sum())} slots; of {tie_slots} adjacent tied slot pairs the library returns "
             f"{lib_ascending} in ascending index order")
     print(line)
-    if os.path.isdir("gpurun_out"):
-        with open("gpurun_out/topk_ties.txt", "w") as f:
+    out_dir = os.environ.get("GCA_TEST_RECORD_DIR")
+    if out_dir and os.path.isdir(out_dir):
+        with open(os.path.join(out_dir, "topk_ties.txt"), "w") as f:
             f.write(line + "\n")
