@@ -182,6 +182,7 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
                     dsA[t4][s] = (__bf16)(st[t4 >> 1][r] * (dpt[t4 >> 1][r] - dsum));
                 }
             if (mult < 0.f) {
+                asm volatile("" ::: "memory");      // keeps this a (uniform, rarely taken) branch instead of 16 masked XORs
 #pragma unroll
                 for (int t4 = 0; t4 < 4; ++t4) dsA[t4] = negate_bf16x8(dsA[t4]);
             }
@@ -443,6 +444,9 @@ gca_bwd_dkdv2_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16
                 dsA[r >> 3][r & 7] = (__bf16)(pw * dp[r]);
             }
             if (wneg) {
+                // a real branch (the empty volatile statement keeps the compiler from turning the block into 32
+                // unconditional XORs with a mask): weights are positive in practice and the branch is uniform
+                asm volatile("" ::: "memory");
 #pragma unroll
                 for (int t2 = 0; t2 < 2; ++t2) { pA[t2] = negate_bf16x8(pA[t2]); dsA[t2] = negate_bf16x8(dsA[t2]); }
             }
@@ -689,6 +693,9 @@ gca_bwd_dkdv_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_
                     dsA[r >> 3][r & 7] = (__bf16)(pw * fmaf(dp[r], p.sm_scale, -d_cur[a][e] * p.sm_scale));
                 }
             if (wneg) {
+                // a real branch (the empty volatile statement keeps the compiler from turning the block into 32
+                // unconditional XORs with a mask): weights are positive in practice and the branch is uniform
+                asm volatile("" ::: "memory");
 #pragma unroll
                 for (int t2 = 0; t2 < 2; ++t2) { pA[t2] = negate_bf16x8(pA[t2]); dsA[t2] = negate_bf16x8(dsA[t2]); }
             }

@@ -122,20 +122,19 @@ struct TileLoader {
     int wave;
     __device__ __forceinline__ TileLoader(int tid, int rs) {
         const int lane = tid & 63;
-        wave = tid >> 6;
+        wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const int row = wave * RPI + lane / PPR;
         const int lp = (lane % PPR) ^ swz(row);
         goff = (unsigned)(row * rs + lp * 8) * 2u;
-        istep = (unsigned)(NW * RPI * rs) * 2u;
+        istep = (unsigned)__builtin_amdgcn_readfirstlane((int)((unsigned)(NW * RPI * rs) * 2u));
     }
     __device__ __forceinline__ void issue(const uint16_t* tile, unsigned char* lds_tile) const {
+        // one vector -> scalar transfer of the tile's address and of the LDS offset; the steps from instruction to
+        // instruction are scalar additions
         const unsigned base = lds_offset_of(lds_tile) + wave * 1024;
+        const unsigned char* sb = (const unsigned char*)uniform_ptr(tile);
 #pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            // the rows of instruction i start i * istep bytes after the tile's first element
-            const void* sb = uniform_ptr((const unsigned char*)tile + (size_t)i * istep);
-            lds_dma_b128(sb, goff, base + i * NW * 1024);
-        }
+        for (int i = 0; i < NI; ++i) lds_dma_b128(sb + (size_t)i * istep, goff, base + i * NW * 1024);
     }
 };
 
