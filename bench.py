@@ -229,7 +229,7 @@ def run_cfg2(torch, dev, seed, sm_n, iters):
         o = gca_hip.attention_indexed(q, ck, cv, idx, w, 0.125, sm_n)
         return torch.autograd.grad(o, (q, ck, cv, w), do)
 
-    t = event_time(torch, step, iters) * 1e-3
+    t = event_time(torch, step, iters, 5) * 1e-3
     _, _, work = cfg2_work()
     out = {"tokens_per_s": round(N * C * S / t, 1), "ms": round(t * 1e3, 4)}
     out.update(bound_of(work["flops"], work["bytes"], t))
@@ -418,9 +418,9 @@ def run_workload(torch, dev, seed, name, quick=False):
     if name == "cfg1_fp32_gpu":
         return run_cfg1_gpu(torch, dev, seed, 5 if quick else 50)
     if name == "cfg2_bf16_sm0":
-        return run_cfg2(torch, dev, seed, 0.0, 3 if quick else 10)
+        return run_cfg2(torch, dev, seed, 0.0, 3 if quick else 20)
     if name == "cfg2_bf16_sm1":
-        return run_cfg2(torch, dev, seed, 1.0, 3 if quick else 10)
+        return run_cfg2(torch, dev, seed, 1.0, 3 if quick else 20)
     if name == "cfg2_bf16_gathered_dropin":
         return run_cfg2_gathered(torch, dev, seed, 3 if quick else 8)
     if name == "cfg3_prefill_1M_fwd":
