@@ -34,8 +34,9 @@
 
 namespace gca {
 
-// references per dkdv workgroup in the indexed form: longer lists are cut into segments of this many
-constexpr int SEG_MAX = 32;
+// references per dkdv workgroup in the indexed form: longer lists are cut into segments of this many (16, 24, 32,
+// 48, 64 and 128 were timed; from 48 on hardly any chunk of the benchmark shapes needs partial tiles)
+constexpr int SEG_MAX = 64;
 
 // Order of the indexed dk/dv workgroups.  All chunks of a (sequence, kv head) pair re-read the same Q / dO rows
 // (those of the pair's later query chunks), K times over.  P pairs are in flight at a time; workgroup b runs on XCD
