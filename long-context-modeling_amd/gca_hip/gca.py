@@ -21,6 +21,7 @@ indices (Z, K) int64 with Z % N == 0.
 """
 from __future__ import annotations
 
+import atexit
 import collections
 import ctypes
 
@@ -176,6 +177,8 @@ class _ListCache:
 
 
 list_cache = _ListCache()
+# the entries hold device tensors and events: release them while the runtime is still up, not during interpreter teardown
+atexit.register(list_cache.clear)
 
 
 def _bwd_indexed(desc, q, k_cache, v_cache, idx, weights, do, lse, dq, dkc, dvc, dw, key_tensor):
