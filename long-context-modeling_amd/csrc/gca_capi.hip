@@ -211,8 +211,8 @@ int lmk_score_topk(const lmk_desc* desc, const void* lmk_q, const void* lmk_k, c
     int rc = check_lmk(desc);
     if (rc != GCA_OK) return rc;
     if (!lmk_q || !lmk_k || !indices || !weights) return GCA_ERR_NULL;
-    // Without a score buffer the fused kernel selects while it scores: 0.81 ms for 16384 x 16384 rows of width 768,
-    // where the two launches take 0.79 ms and write and re-read the 0.5 GB matrix.  Its workgroups walk their
+    // Without a score buffer the fused kernel selects while it scores: 0.80 ms for 16384 x 16384 rows of width 768,
+    // where the two launches take 0.62 ms and write and re-read the 0.5 GB matrix.  Its workgroups walk their
     // blocks one by one, which hides memory latency less well than the score kernel's 16K independent blocks, so
     // a caller that wants the scores anyway gets the two launches.
     if (scores == nullptr) {

@@ -81,8 +81,8 @@ def landmark_score_topk(lmk_q, lmk_k, topk, hidden_size=None, causal=True, noise
     """Scoring and selection through the one-call entry point ``lmk_score_topk`` (model/DRT.py:612-627).
     Returns (scores or None, indices, weights).  With ``return_scores=False`` and a score matrix of at least
     ``FUSED_MIN_BYTES`` (2 GiB) the matrix is never written: the fused kernel (bf16, width a multiple of 64, at
-    least 32 query rows, k <= 32) selects while it scores.  It is the slower of the two forms (0.8-1.1 ms against
-    0.8 ms for 16384 x 16384 rows; the memory is what it saves), so smaller requests and shapes it does not take go
+    least 32 query rows, k <= 32) selects while it scores.  It is the slower of the two forms (0.80 ms against
+    0.62 ms for 16384 x 16384 rows; the memory is what it saves), so smaller requests and shapes it does not take go
     through ``landmark_scores`` + ``landmark_topk`` and drop the scores afterwards.  ``fused=True`` / ``False``
     overrides the size rule."""
     assert lmk_q.is_cuda and lmk_q.dim() == 3 and lmk_k.dim() == 3 and lmk_q.dtype in _DT and lmk_k.dtype == lmk_q.dtype
