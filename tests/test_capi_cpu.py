@@ -181,3 +181,36 @@ def test_header_is_c99_and_links_from_plain_c(tmp_path):
     assert "gca_fwd(NULL desc) -> 1" in out and "gca_fwd(bad heads) -> 2" in out
     assert "bwd workspace for a bad descriptor: 0" in out
     assert "lmk_score(C > E) -> 2" in out and "chunk_cache_append(overflow) -> 2" in out
+
+
+def test_validation_of_the_list_fused_and_static_entry_points():
+    """Argument checks answer before anything touches a GPU: NULL pointers, missing or short buffers, requests the
+    fused kernel or the static scratch cannot take."""
+    L = _lib.lib()
+    one = ctypes.c_void_p(16)   # never dereferenced: validation fails first
+    null = ctypes.c_void_p(0)
+    d = _desc(N=2, C=2)          # indexed form: Z = 2 rows, one per sequence
+    need = L.gca_lists_workspace_bytes(ctypes.byref(d))
+    assert need > 0
+    assert L.gca_lists_build(ctypes.byref(d), null, one, need, null) == 1
+    assert L.gca_lists_build(ctypes.byref(d), one, null, need, null) == 5
+    assert L.gca_lists_build(ctypes.byref(d), one, one, need - 1, null) == 5
+    assert L.gca_bwd_indexed_lists(ctypes.byref(d), one, one, one, one, one, one, one, one, one, one, one, null, 0, one,
+                                   need, null) == 5                                      # no workspace
+    assert L.gca_lists_workspace_bytes(ctypes.byref(_desc(N=3, C=4))) == 0                # Z % N != 0
+
+    fp32 = _lib.LmkDesc(dtype=0, topk=8, N=1, C=64, E=64, Dm=64, causal=1, hidden_size=64.0)
+    assert L.lmk_score_topk(ctypes.byref(fp32), one, one, null, null, one, one, null, 0, null) == _lib.GCA_ERR_UNSUPPORTED
+    assert L.lmk_score_topk(ctypes.byref(fp32), one, one, null, null, null, one, null, 0, null) == 1
+    odd = _lib.LmkDesc(dtype=1, topk=8, N=1, C=64, E=64, Dm=40, causal=1, hidden_size=40.0)    # width not a multiple of 64
+    assert L.lmk_score_topk(ctypes.byref(odd), one, one, null, null, one, one, null, 0, null) == _lib.GCA_ERR_UNSUPPORTED
+    big_k = _lib.LmkDesc(dtype=1, topk=64, N=1, C=64, E=4096, Dm=64, causal=1, hidden_size=64.0)
+    assert L.lmk_score_topk(ctypes.byref(big_k), one, one, null, null, one, one, null, 0, null) == _lib.GCA_ERR_UNSUPPORTED
+    long_rows = _lib.LmkDesc(dtype=1, topk=8, N=1, C=4096, E=4096, Dm=64, causal=1, hidden_size=64.0)
+    assert L.lmk_topk_workspace_bytes(ctypes.byref(long_rows)) >= 4096 * 4 * 8 * 8        # segment winners of the fused form
+    assert L.lmk_score_topk(ctypes.byref(long_rows), one, one, null, null, one, one, null, 0, null) == 5
+
+    too_big = _lib.LmkDesc(dtype=1, topk=8, N=64, C=64, E=4096, Dm=64, causal=1, hidden_size=64.0)   # 32 MiB of scores
+    assert L.lmk_score_topk_static(ctypes.byref(too_big), one, one, null, one, one, null) == _lib.GCA_ERR_SCRATCH_LIMIT
+    assert L.lmk_score_topk_static(ctypes.byref(too_big), null, one, null, one, one, null) == 1
+    assert b"scratch" in L.gca_strerror(_lib.GCA_ERR_SCRATCH_LIMIT).lower()
