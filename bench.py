@@ -376,6 +376,36 @@ def run_cfg5(torch, dev, seed, which, iters):
     return out
 
 
+def oracle_eager_on_gpu(torch, iters=3):
+    """A second baseline beside the CPU one: the same oracle (the formulation the reference uses as its own check,
+    ltriton/gca.py:912-921 + autograd, with its retrieval and gather, model/DRT.py:612-627, :193-200) run as eager
+    torch ops on this GPU, at config 2 in fp32 -- what the path costs here without hand-written kernels."""
+    from oracle import gca_oracle as orc
+    dev = torch.device("cuda:0")
+    try:
+        N, C, H, S, d, K = 8, 256, 12, 64, 64, 8
+        g = torch.Generator(device=dev).manual_seed(99)
+        q_all = (torch.randn(N, C, H, S, d, device=dev, generator=g) * 0.5).requires_grad_(True)
+        ck = (torch.randn(N, C, S, H * d, device=dev, generator=g) * 0.5).requires_grad_(True)
+        cv = (torch.randn(N, C, S, H * d, device=dev, generator=g) * 0.5).requires_grad_(True)
+        lq = torch.randn(N, C, H * d, device=dev, generator=g)
+        lk = torch.randn(N, C, H * d, device=dev, generator=g)
+        do = torch.randn(N, C, H, S, d, device=dev, generator=g)
+
+        def step():
+            out, _, _ = orc.gca_layer(q_all, ck, cv, lq, lk, K, H, sm_n=1.0)
+            torch.autograd.grad(out, (q_all, ck, cv), do)
+
+        t = event_time(torch, step, iters, 1) * 1e-3
+        del q_all, ck, cv, lq, lk, do
+        torch.cuda.empty_cache()
+        return {"tokens_per_s": round(N * C * S / t, 1), "ms_per_step": round(t * 1e3, 2),
+                "config": "config 2 shapes (B=8 H=12 d=64 L=16384 chunk=64 top-k=8), fp32, eager torch ops"}
+    except Exception as exc:                                   # e.g. out of memory on a smaller GPU: the line is optional
+        torch.cuda.empty_cache()
+        return {"error": type(exc).__name__}
+
+
 def cpu_baseline(torch, budget_s=12.0):
     """CPU oracle at BASELINE.json config 1 (fp32, B=2, H=4, d=64, L=1024, chunk 64, top-k 4, softmax1 on):
     retrieval + forward + autograd backward, median over the iterations that fit the budget."""
@@ -403,7 +433,11 @@ def cpu_baseline(torch, budget_s=12.0):
         ts.append(time.perf_counter() - t0)
     ts.sort()
     med = ts[len(ts) // 2]
-    return {"value": N * C * S / med, "unit": "tokens/s", "cores": threads, "kind": "port",
+    eager = None
+    if torch.cuda.is_available():
+        eager = oracle_eager_on_gpu(torch)
+    return {"same_formulation_torch_eager_on_gpu": eager,
+            "value": N * C * S / med, "unit": "tokens/s", "cores": threads, "kind": "port",
             "sample": f"config 1 (fp32 B=2 H=4 d=64 L=1024 chunk=64 top-k=4), median of {len(ts)} fwd+bwd steps, "
                       f"{med * 1e3:.2f} ms/step, {threads} torch threads on a host reporting os.cpu_count()="
                       f"{os.cpu_count()}, torch {torch.__version__}"}
@@ -519,6 +553,9 @@ def main():
                 "algorithmic_GFLOP_per_launch": b["algorithmic_GFLOP"], "compulsory_GB_per_launch": b["compulsory_GB"],
                 "frac_of_mfma_peak": b["frac_of_mfma_peak"], "frac_of_hbm_peak": b["frac_of_hbm_peak"],
                 "kernel_ms": {k_: round(v, 4) for k_, v in kt.items()},
+                "stage_ms": {"retrieval": round(t_retr, 4), "forward": round(kt["gca_fwd_mfma_kernel"], 4),
+                             "backward": round(sum(v for k_, v in kt.items() if k_ != "gca_fwd_mfma_kernel"), 4),
+                             "sum": round(t_retr + sum(kt.values()), 4), "step": round(dt * 1e3, 4)},
                 "per_kernel_frac": {k_: bound_of(per_kernel[k_]["flops"], per_kernel[k_]["bytes"], kt[k_] * 1e-3)["frac"]
                                     for k_ in per_kernel},
                 "simd_time_share": {"note": "matrix and vector instructions do not overlap on a SIMD of this GPU (measured: "

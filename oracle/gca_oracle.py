@@ -69,15 +69,15 @@ def landmark_scores(lmk_q: torch.Tensor, lmk_k: torch.Tensor, hidden_size: Optio
     return torch.einsum('ncd,ned->nce', lmk_q, lmk_k) / math.sqrt(hidden_size)
 
 
-def causal_visible(dec_chunk_num: int, enc_chunk_num: int, max_chunk_win: int = -1) -> torch.Tensor:
+def causal_visible(dec_chunk_num: int, enc_chunk_num: int, max_chunk_win: int = -1, device=None) -> torch.Tensor:
     """Boolean (dec, enc) matrix, True where a decoder row may see an encoder chunk.
 
     model/DRT.py:596-603: decoder ids are the LAST ``dec_chunk_num`` of
     ``arange(enc_chunk_num)``; visible iff ``dec_id > enc_id`` (strictly past),
     optionally also ``dec_id <= enc_id + max_chunk_win``.
     """
-    dec = torch.arange(enc_chunk_num)[-dec_chunk_num:] if dec_chunk_num > 0 else torch.arange(0)
-    enc = torch.arange(enc_chunk_num)
+    dec = torch.arange(enc_chunk_num, device=device)[-dec_chunk_num:] if dec_chunk_num > 0 else torch.arange(0, device=device)
+    enc = torch.arange(enc_chunk_num, device=device)
     vis = dec.unsqueeze(1) > enc.unsqueeze(0)
     if max_chunk_win != -1:
         vis = vis & (dec.unsqueeze(1) <= enc.unsqueeze(0) + max_chunk_win)
@@ -86,7 +86,7 @@ def causal_visible(dec_chunk_num: int, enc_chunk_num: int, max_chunk_win: int = 
 
 def mask_scores(scores: torch.Tensor, max_chunk_win: int = -1) -> torch.Tensor:
     """Fill the non-visible entries with -inf   (model/DRT.py:613)."""
-    vis = causal_visible(scores.shape[1], scores.shape[2], max_chunk_win)
+    vis = causal_visible(scores.shape[1], scores.shape[2], max_chunk_win, scores.device)
     return scores.masked_fill(~vis, float('-inf'))
 
 
@@ -134,7 +134,7 @@ def gather_chunks(chunk_k: torch.Tensor, chunk_v: torch.Tensor, indices: torch.T
     K = indices.shape[-1]
     d = Dm // num_kv_heads
     idx = indices[:, :-1, :].reshape(N, (C - 1) * K)
-    bidx = torch.arange(N).unsqueeze(1)
+    bidx = torch.arange(N, device=chunk_k.device).unsqueeze(1)
     k = chunk_k[bidx, idx]                                       # (N, (C-1)K, S, Dm)
     v = chunk_v[bidx, idx]
     k = k.reshape(N, C - 1, K, S, num_kv_heads, d).permute(0, 1, 4, 2, 3, 5).reshape(N * (C - 1), num_kv_heads, K, S, d)
@@ -285,6 +285,6 @@ def gca_module_forward(hidden, chunk_k, chunk_v, indices, weights, norm_w, eps, 
     vals = gca_forward(q, k, v, w, 1.0 / math.sqrt(d), sm_n if sm_n_functional else 0.0)   # ((N D), h, S, d)
     vals = vals.reshape(N, C - 1, num_heads, S, d).permute(0, 1, 3, 2, 4).reshape(N, (C - 1) * S, num_heads * d)
     o = F.linear(vals, wo, bo)
-    ret = torch.zeros((N, C * S, dim), dtype=o.dtype)
+    ret = torch.zeros((N, C * S, dim), dtype=o.dtype, device=o.device)
     ret[:, -o.shape[1]:, :] = o                                         # model/DRT.py:387-394
     return ret
