@@ -1433,6 +1433,86 @@ lmk_bwd_dk_kernel(lmk_desc d, int kk, const T* __restrict__ lq, const float* __r
     }
 }
 
+// Small problems (C * kk <= LMK_BWD_SEARCH_MAX): two launches instead of eight, no ds buffer and no lists.  The
+// gather kernel computes its row's ds itself; the landmark kernel finds its references by scanning the sequence's
+// C * kk indices (32 KB at 256 chunks, k = 8) and keeps them in ascending order, which is the order of the list
+// version -- the sums are the same bits.
+constexpr int LMK_BWD_SEARCH_MAX = 32768;
+constexpr int LMK_BWD_SEARCH_REFS = 4096;      // a landmark is referenced at most once per row: C <= 4096 here
+
+__device__ __forceinline__ float lmk_ds_of(const lmk_desc& d, int kk, const float* __restrict__ w,
+                                           const float* __restrict__ dw, int64_t row, int k) {
+    float dot = 0.f;
+    for (int j = 0; j < kk; ++j) dot += w[row * kk + j] * dw[row * kk + j];
+    const float inv = 1.f / sqrtf(d.hidden_size);
+    return w[row * kk + k] * (dw[row * kk + k] - dot) * inv;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+lmk_bwd_dq_fused_kernel(lmk_desc d, int kk, const T* __restrict__ lk, const int64_t* __restrict__ idx,
+                        const float* __restrict__ w, const float* __restrict__ dw, T* __restrict__ dlq) {
+    __shared__ float s_ds[TOPK_MAX_KP];
+    __shared__ int64_t s_e[TOPK_MAX_KP];
+    const int64_t row = blockIdx.x;
+    const int64_t n = row / d.C;
+    if ((int)threadIdx.x < kk) {
+        s_ds[threadIdx.x] = lmk_ds_of(d, kk, w, dw, row, threadIdx.x);
+        s_e[threadIdx.x] = clamp_idx(idx[row * kk + threadIdx.x], d.E);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < d.Dm; i += 256) {
+        float acc = 0.f;
+        for (int k = 0; k < kk; ++k) {
+            const float g = s_ds[k];
+            if (g != 0.f) acc = fmaf(g, to_f(lk[(n * d.E + s_e[k]) * d.Dm + i]), acc);
+        }
+        dlq[row * d.Dm + i] = from_f<T>(acc);
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+lmk_bwd_dk_search_kernel(lmk_desc d, int kk, const T* __restrict__ lq, const int64_t* __restrict__ idx,
+                         const float* __restrict__ w, const float* __restrict__ dw, T* __restrict__ dlk) {
+    __shared__ int s_ref[LMK_BWD_SEARCH_REFS];
+    __shared__ float s_g[LMK_BWD_SEARCH_REFS];
+    __shared__ int s_wcnt[4];
+    __shared__ int s_total;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t ce = blockIdx.x;                 // n * E + e
+    const int64_t n = ce / d.E, e = ce % d.E;
+    const int per_seq = (int)d.C * kk;
+    const int64_t* seq = idx + n * per_seq;
+    if (tid == 0) s_total = 0;
+    __syncthreads();
+    // ordered compaction of the matching positions, 256 at a time
+    for (int base = 0; base < per_seq; base += 256) {
+        const int pos = base + tid;
+        const bool hit = pos < per_seq && clamp_idx(seq[pos], d.E) == e;
+        const uint64_t m = __ballot(hit);
+        if (lane == 0) s_wcnt[wave] = __popcll(m);
+        __syncthreads();
+        int off = s_total;
+        for (int wv = 0; wv < wave; ++wv) off += s_wcnt[wv];
+        if (hit) {
+            const int at = off + __popcll(m & ((1ull << lane) - 1ull));
+            const int64_t row = n * d.C + pos / kk;
+            s_ref[at] = (int)(n * per_seq + pos);
+            s_g[at] = lmk_ds_of(d, kk, w, dw, row, pos % kk);
+        }
+        __syncthreads();
+        if (tid == 0) s_total += s_wcnt[0] + s_wcnt[1] + s_wcnt[2] + s_wcnt[3];
+        __syncthreads();
+    }
+    const int cnt = s_total;
+    for (int i = tid; i < d.Dm; i += 256) {
+        float acc = 0.f;
+        for (int r = 0; r < cnt; ++r) acc = fmaf(s_g[r], to_f(lq[(int64_t)(s_ref[r] / kk) * d.Dm + i]), acc);
+        dlk[ce * d.Dm + i] = from_f<T>(acc);
+    }
+}
+
 static Params lists_params(const lmk_desc& d, int kk) {
     Params p = {};
     p.Z = d.N * d.C; p.K = kk; p.N = d.N; p.C = d.E; p.zpn = d.C; p.indexed = 1;
@@ -1452,6 +1532,12 @@ static int launch_lmk_bwd_t(const lmk_desc& d, int kk, const void* lq, const voi
                             const float* w, const float* dw, void* dlq, void* dlk, void* wsp, hipStream_t s) {
     const int64_t R = d.N * d.C;
     if (R > 0x7fffffffLL || d.N * d.E > 0x7fffffffLL) return GCA_ERR_SHAPE;
+    if (d.C * kk <= LMK_BWD_SEARCH_MAX && d.C <= LMK_BWD_SEARCH_REFS && R * kk <= 0x7fffffffLL) {
+        hipLaunchKernelGGL((lmk_bwd_dq_fused_kernel<T>), dim3((unsigned)R), dim3(256), 0, s, d, kk, (const T*)lk, idx, w, dw, (T*)dlq);
+        hipLaunchKernelGGL((lmk_bwd_dk_search_kernel<T>), dim3((unsigned)(d.N * d.E)), dim3(256), 0, s, d, kk, (const T*)lq, idx, w,
+                           dw, (T*)dlk);
+        return hipGetLastError() == hipSuccess ? GCA_OK : GCA_ERR_LAUNCH;
+    }
     float* ds = (float*)wsp;
     const size_t dsb = ((size_t)R * kk * sizeof(float) + 255) / 256 * 256;
     const Params p = lists_params(d, kk);

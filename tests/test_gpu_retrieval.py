@@ -168,10 +168,12 @@ def test_gca_layer_end_to_end_fp32():
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
-def test_weights_backward_to_landmarks(dtype, tol):
-    # dw -> softmax -> gather -> scores -> both landmark embeddings (autograd of model/DRT.py:612, :626-627)
+@pytest.mark.parametrize("N,C,Dm,K", [(3, 40, 256, 4), (2, 300, 64, 8), (1, 4200, 64, 8)])
+def test_weights_backward_to_landmarks(N, C, Dm, K, dtype, tol):
+    # dw -> softmax -> gather -> scores -> both landmark embeddings (autograd of model/DRT.py:612, :626-627).
+    # Up to 4096 rows the landmark gradient finds its references by scanning the indices, above that through
+    # the reference lists: the last shape takes the lists.
     import gca_hip
-    N, C, Dm, K = 3, 40, 256, 4
     lq, lk = gen((N, C, Dm), 71, 1.0, dtype), gen((N, C, Dm), 72, 1.0, dtype)
     dw = gen((N, C, K), 73, 1.0, torch.float32)
     lqr, lkr = lq.double().requires_grad_(True), lk.double().requires_grad_(True)
