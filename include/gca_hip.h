@@ -104,14 +104,16 @@ typedef struct lmk_desc {
     int64_t C;              /* query landmarks (rows) per sequence */
     int64_t E;              /* candidate chunks per sequence */
     int32_t Dm;             /* landmark width */
-    int32_t causal;         /* 1: row c sees chunk e iff (E - C + c) > e, others are -inf.  This is
-                               _enc_dec_score_mask with max_chunk_win = -1 (model/DRT.py:590-607), the only value
-                               the reference's retrieval passes (:613, :840 call it with the default); the
-                               sliding-window variant (max_chunk_win >= 0) is not implemented */
+    int32_t causal;         /* 1: row c sees chunk e iff (E - C + c) > e, others are -inf: _enc_dec_score_mask
+                               (model/DRT.py:590-607) as the reference's retrieval applies it (:613, :840) */
     float hidden_size;      /* scores are divided by sqrt(hidden_size) */
     int32_t lmk_k_rows;     /* landmark rows allocated per sequence in lmk_k: sequence n starts at row
                                n * lmk_k_rows (a cache with spare capacity); 0 means E (dense).  Honoured by
                                lmk_score and lmk_score_topk; lmk_weights_bwd needs the dense form */
+    int32_t chunk_win;      /* 0: no window, the reference's max_chunk_win = -1.  w > 0 (with causal): row c sees
+                               chunk e only if also e >= (E - C + c) - w, the w most recent of its visible chunks:
+                               max_chunk_win = w (model/DRT.py:601-603).  Masked chunks on either side tie at -inf
+                               and fill the slots of a row that sees fewer than k chunks lowest index first */
 } lmk_desc;
 
 /* What chunk_cache_append does with the last row of every chunk it stores (the landmark position). */
@@ -134,7 +136,7 @@ typedef struct chunk_cache_desc {
     int32_t reserved;
 } chunk_cache_desc;
 
-/* Library version (major*10000 + minor*100 + patch) and status text. */
+/* Library version (major*10000 + minor*100 + patch; 200: lmk_desc has chunk_win) and status text. */
 int gca_version(void);
 const char* gca_strerror(int status);
 

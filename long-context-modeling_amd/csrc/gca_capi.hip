@@ -43,6 +43,7 @@ int check_lmk(const lmk_desc* d) {
     if (d->E > INT32_MAX) return GCA_ERR_SHAPE;
     if (d->lmk_k_rows != 0 && d->lmk_k_rows < d->E) return GCA_ERR_SHAPE;
     if (d->causal && d->C > d->E) return GCA_ERR_SHAPE;
+    if (d->chunk_win < 0) return GCA_ERR_SHAPE;
     if (!(d->hidden_size > 0.f)) return GCA_ERR_SHAPE;
     return GCA_OK;
 }
@@ -79,7 +80,7 @@ size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 
 extern "C" {
 
-int gca_version(void) { return 100; }
+int gca_version(void) { return 200; }
 
 const char* gca_strerror(int status) {
     switch (status) {

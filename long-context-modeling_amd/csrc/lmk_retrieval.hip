@@ -53,6 +53,29 @@ template <> __device__ __forceinline__ float finish_score<bf16_t>(float dot, flo
     return bf16_round(q);
 }
 
+// The mask of model/DRT.py:599-603 for query landmark c: candidate e is visible iff lo <= e < hi, where
+// hi = E - C + c (strict past) and lo = hi - chunk_win when a window is set (max_chunk_win = chunk_win).
+struct VisibleRange {
+    int64_t lo, hi;
+    __device__ __forceinline__ bool has(int64_t e) const { return e < hi && e >= lo; }
+};
+__device__ __forceinline__ VisibleRange visible_range(const lmk_desc& d, int64_t c) {
+    VisibleRange v;
+    v.hi = d.causal ? d.E - d.C + c : d.E;
+    v.lo = (d.causal && d.chunk_win > 0) ? v.hi - d.chunk_win : INT64_MIN;
+    return v;
+}
+__device__ __forceinline__ bool row_sees(const lmk_desc& d, int64_t c, int64_t e) { return visible_range(d, c).has(e); }
+// The same in block-relative 32-bit form: with vis0 = block_vis0(d, c0, e0) and win0 = block_win0(d, c0, e0), column
+// el of row rl (both below 4096) is visible iff win0 + rl <= el < vis0 + rl.
+__device__ __forceinline__ int block_vis0(const lmk_desc& d, int64_t c0, int64_t e0) {
+    return d.causal ? (int)max((int64_t)-4096, min((int64_t)4096, d.E - d.C + c0 - e0)) : 4096;
+}
+__device__ __forceinline__ int block_win0(const lmk_desc& d, int64_t c0, int64_t e0) {
+    return (d.causal && d.chunk_win > 0)
+               ? (int)max((int64_t)-8192, min((int64_t)4096, d.E - d.C + c0 - e0 - d.chunk_win)) : -8192;
+}
+
 // One wavefront per candidate landmark e; all C (<= SCAN_MAX_C) query rows of the sequence
 // sit in LDS as floats.  Requires Dm % (16 / sizeof(T)) == 0.
 constexpr int SCAN_MAX_C = 4;
@@ -120,7 +143,7 @@ lmk_score_scan_kernel(lmk_desc d, const T* __restrict__ lq, const T* __restrict_
                 const int64_t e = e0 + a;
                 if (lane == 0 && e < d.E) {
                     float r = finish_score<T>(x, sqrt_hidden);
-                    if (d.causal && !((d.E - C + c) > e)) r = -INFINITY;
+                    if (!row_sees(d, c, e)) r = -INFINITY;
                     scores[(n * C + c) * d.E + e] = from_f<T>(r);
                 }
             }
@@ -180,12 +203,15 @@ lmk_score_scan_mfma_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const ui
         }
         // register r is query row 8*(r/4) + 4*h + r%4, column = landmark e0 + n32
         const int64_t e = e0 + n32;
+        // visible iff rel < c and rel + window >= c; both sides moved so that the row enters as a constant of r
+        const int64_t rel = d.causal ? e - (d.E - C) - 4 * h : INT64_MIN / 2;
+        const int64_t relw = (d.causal && d.chunk_win > 0) ? rel + d.chunk_win : INT64_MAX / 2;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int c = 8 * (r >> 2) + 4 * h + (r & 3);
             if (c < C && e < d.E) {
                 float x = finish_score<bf16_t>(acc[r], sqrt_hidden);
-                if (d.causal && !((d.E - C + c) > e)) x = -INFINITY;
+                if (!(rel < 8 * (r >> 2) + (r & 3) && relw >= 8 * (r >> 2) + (r & 3))) x = -INFINITY;
                 scores[(nb * C + c) * d.E + e] = f_to_bf16_bits(x);
             }
         }
@@ -281,7 +307,7 @@ lmk_score_mfma64_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const uint1
     f32x16 acc[2];
     score_block_mfma(d, lq + (nb * d.C + c0) * d.Dm, lk + (nb * d.lmk_k_rows + e0) * d.Dm, crows, d.E - e0, smem, acc);
     const float sqrt_hidden = sqrtf(d.hidden_size);
-    const int vis0 = d.causal ? (int)max((int64_t)-4096, min((int64_t)4096, off + c0 - e0)) : 4096;
+    const int vis0 = block_vis0(d, c0, e0), win0 = block_win0(d, c0, e0);
     uint16_t* lane_out = scores + (nb * d.C + c0 + 32 * wr + 4 * h) * d.E + e0 + 64 * wc + n32;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -291,7 +317,7 @@ lmk_score_mfma64_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const uint1
         for (int t = 0; t < 2; ++t) {
             const int el = 64 * wc + 32 * t + n32;
             if (rl < crows && el < erows) {
-                const float x = (el < vis0 + rl) ? finish_score<bf16_t>(acc[t][r], sqrt_hidden) : -INFINITY;
+                const float x = (el < vis0 + rl && el >= win0 + rl) ? finish_score<bf16_t>(acc[t][r], sqrt_hidden) : -INFINITY;
                 row_out[32 * t] = f_to_bf16_bits(x);
             }
         }
@@ -380,9 +406,9 @@ lmk_score_mfma_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const uint16_
         wait_async_tiles();
         __syncthreads();
     }
-    // epilogue in block-relative 32-bit coordinates: row rl, column el; visible iff el < vis0 + rl
+    // epilogue in block-relative 32-bit coordinates: row rl, column el; visible iff win0 + rl <= el < vis0 + rl
     const float sqrt_hidden = sqrtf(d.hidden_size);
-    const int vis0 = d.causal ? (int)max((int64_t)-4096, min((int64_t)4096, off + c0 - e0)) : 4096;
+    const int vis0 = block_vis0(d, c0, e0), win0 = block_win0(d, c0, e0);
     uint16_t* lane_out = scores + (nb * d.C + c0 + 64 * wr + 4 * h) * d.E + e0 + 64 * wc + n32;
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt)
@@ -394,7 +420,8 @@ lmk_score_mfma_kernel(lmk_desc d, const uint16_t* __restrict__ lq, const uint16_
             for (int ct = 0; ct < 2; ++ct) {
                 const int el = 64 * wc + 32 * ct + n32;
                 if (rl < crows && el < erows) {
-                    const float x = (el < vis0 + rl) ? finish_score<bf16_t>(acc[rt][ct][r], sqrt_hidden) : -INFINITY;
+                    const float x = (el < vis0 + rl && el >= win0 + rl) ? finish_score<bf16_t>(acc[rt][ct][r], sqrt_hidden)
+                                                                        : -INFINITY;
                     row_out[32 * ct] = f_to_bf16_bits(x);
                 }
             }
@@ -444,7 +471,7 @@ lmk_score_tile_kernel(lmk_desc d, const T* __restrict__ lq, const T* __restrict_
             const int64_t c = c0 + ty * 2 + i, e = e0 + tx * 2 + jx;
             if (c < d.C && e < d.E) {
                 float r = finish_score<T>(acc[i][jx], sqrt_hidden);
-                if (d.causal && !((off + c) > e)) r = -INFINITY;
+                if (!visible_range(d, c).has(e)) r = -INFINITY;
                 scores[(n * d.C + c) * d.E + e] = from_f<T>(r);
             }
         }
@@ -688,13 +715,13 @@ template <> __device__ __forceinline__ float round_like<bf16_t>(float x) { retur
 
 // softmax over the kk selected noise-free masked scores; NaN (all -inf) -> 0
 template <typename T>
-__device__ void emit_row(const lmk_desc& d, const uint64_t* keys, int kk, int64_t row, int64_t limit,
+__device__ void emit_row(const lmk_desc& d, const uint64_t* keys, int kk, int64_t row, const VisibleRange& vr,
                          const T* __restrict__ scores, int64_t* __restrict__ indices, float* __restrict__ weights,
                          float* sval, int tid) {
     if (tid < kk) {
         const uint32_t e = key_index(keys[tid]);
         float sc = to_f(scores[row * d.E + e]);
-        if (d.causal && !((int64_t)e < limit)) sc = -INFINITY;
+        if (!vr.has((int64_t)e)) sc = -INFINITY;
         sval[tid] = sc;
         indices[row * kk + tid] = (int64_t)e;
     }
@@ -724,7 +751,8 @@ lmk_topk_kernel(lmk_desc d, int kk, int kp, int nseg, int64_t seg_len, int64_t r
     const int seg = blockIdx.x;
     const int64_t row = row0 + blockIdx.y;
     const int64_t c = row % d.C;
-    const int64_t limit = d.causal ? (d.E - d.C + c) : d.E;      // candidates e < limit are visible
+    const VisibleRange vr = visible_range(d, c);
+    const int64_t limit = vr.hi;
     // masked candidates all tie at -inf and rank by index, so only the first kk of the row matter
     const int64_t scan_end = min(d.E, max(limit, (int64_t)kk));
     const int64_t lo = (int64_t)seg * seg_len;
@@ -740,7 +768,7 @@ lmk_topk_kernel(lmk_desc d, int kk, int kp, int nseg, int64_t seg_len, int64_t r
             if (e < hi) {
                 float sv = to_f(scores[row * d.E + e]);
                 if (noise != nullptr) sv = round_like<T>(sv + to_f(noise[row * d.E + e]));
-                if (d.causal && !(e < limit)) sv = -INFINITY;
+                if (!vr.has(e)) sv = -INFINITY;
                 key = make_key(sv, (uint32_t)e);
             }
             keys[carry + i] = key;
@@ -751,7 +779,7 @@ lmk_topk_kernel(lmk_desc d, int kk, int kp, int nseg, int64_t seg_len, int64_t r
     } while (pos < hi);
 
     if (nseg == 1) {
-        emit_row<T>(d, keys, kk, row, limit, scores, indices, weights, sval, tid);
+        emit_row<T>(d, keys, kk, row, vr, scores, indices, weights, sval, tid);
     } else if (tid < kp) {
         ws[(row * nseg + seg) * kp + tid] = keys[tid];
     }
@@ -766,7 +794,7 @@ lmk_topk_merge_kernel(lmk_desc d, int kk, int kp, int nseg, int64_t row0, const 
     const int tid = threadIdx.x;
     const int64_t row = row0 + blockIdx.x;
     const int64_t c = row % d.C;
-    const int64_t limit = d.causal ? (d.E - d.C + c) : d.E;
+    const VisibleRange vr = visible_range(d, c);
     const int64_t total = (int64_t)nseg * kp;
     int carry = 0;
     int64_t pos = 0;
@@ -780,7 +808,7 @@ lmk_topk_merge_kernel(lmk_desc d, int kk, int kp, int nseg, int64_t row0, const 
         carry = kp;
         pos += take;
     } while (pos < total);
-    emit_row<T>(d, keys, kk, row, limit, scores, indices, weights, sval, tid);
+    emit_row<T>(d, keys, kk, row, vr, scores, indices, weights, sval, tid);
 }
 
 // Tournament version of the two kernels above for kp <= 32.  A tile is TOPK_THREADS * KP candidates.
@@ -797,7 +825,8 @@ lmk_topk_reg_kernel(lmk_desc d, int kk, int nseg, int64_t seg_len, int64_t row0,
     const int seg = blockIdx.x;
     const int64_t row = row0 + blockIdx.y;
     const int64_t c = row % d.C;
-    const int64_t limit = d.causal ? (d.E - d.C + c) : d.E;
+    const VisibleRange vr = visible_range(d, c);
+    const int64_t limit = vr.hi;
     const int64_t scan_end = min(d.E, max(limit, (int64_t)kk));
     const int64_t lo = (int64_t)seg * seg_len;
     const int64_t hi = min(lo + seg_len, scan_end);
@@ -842,7 +871,7 @@ lmk_topk_reg_kernel(lmk_desc d, int kk, int nseg, int64_t seg_len, int64_t row0,
                     if (e < hi) {
                         float sv = to_f(sc.t[j]);
                         if (noise != nullptr) sv = round_like<T>(sv + to_f(nz.t[j]));
-                        if (d.causal && !(e < limit)) sv = -INFINITY;
+                        if (!vr.has(e)) sv = -INFINITY;
                         key = SegKey<T>::make(sv, e, lo);
                     }
                     if (v * VN + j < KP) a[v * VN + j] = key;
@@ -856,7 +885,7 @@ lmk_topk_reg_kernel(lmk_desc d, int kk, int nseg, int64_t seg_len, int64_t row0,
                 if (e < hi) {
                     float sv = to_f(srow[e]);
                     if (noise != nullptr) sv = round_like<T>(sv + to_f(nrow[e]));
-                    if (d.causal && !(e < limit)) sv = -INFINITY;
+                    if (!vr.has(e)) sv = -INFINITY;
                     key = SegKey<T>::make(sv, e, lo);
                 }
                 a[i] = key;
@@ -907,7 +936,7 @@ lmk_topk_reg_kernel(lmk_desc d, int kk, int nseg, int64_t seg_len, int64_t row0,
         for (int i = 0; i < KP; ++i) win[i] = SegKey<T>::global(best[i], lo);
     __syncthreads();
     if (nseg == 1) {
-        emit_row<T>(d, win, kk, row, limit, scores, indices, weights, sval, tid);
+        emit_row<T>(d, win, kk, row, vr, scores, indices, weights, sval, tid);
     } else if (tid < KP) {
         ws[(row * nseg + seg) * KP + tid] = win[tid];
     }
@@ -923,7 +952,7 @@ lmk_topk_reg_merge_kernel(lmk_desc d, int kk, int nseg, int64_t row0, const T* _
     const int tid = threadIdx.x;
     const int64_t row = row0 + blockIdx.x;
     const int64_t c = row % d.C;
-    const int64_t limit = d.causal ? (d.E - d.C + c) : d.E;
+    const VisibleRange vr = visible_range(d, c);
     // each segment's KP winners are already sorted descending: a thread takes whole segments
     uint64_t best[KP];
 #pragma unroll
@@ -939,7 +968,7 @@ lmk_topk_reg_merge_kernel(lmk_desc d, int kk, int nseg, int64_t row0, const T* _
 #pragma unroll
         for (int i = 0; i < KP; ++i) win[i] = best[i];
     __syncthreads();
-    emit_row<T>(d, win, kk, row, limit, scores, indices, weights, sval, tid);
+    emit_row<T>(d, win, kk, row, vr, scores, indices, weights, sval, tid);
 }
 
 static int next_pow2(int x) { int p = 1; while (p < x) p <<= 1; return p; }
@@ -1153,9 +1182,10 @@ lmk_score_topk_fused_kernel(lmk_desc d, int kk, int nseg, int64_t seg_len, const
         f32x16 acc[2];
         score_block_mfma(d, lq + (nb * d.C + c0) * d.Dm, lk + (nb * d.lmk_k_rows + e0) * d.Dm, crows, d.E - e0, smem, acc);
         // block-relative 32-bit coordinates: row rl = 32*wr + 8*(r/4) + 4*h + r%4, column el = 64*wc + 32*t + n32.
-        // visible: el < vis0 + rl; candidate: el < min(erows, max(vis0 + rl, kk - e0)); all bounds fit an int.
+        // visible: win0 + rl <= el < vis0 + rl; candidate: el < min(erows, max(vis0 + rl, kk - e0)) (columns below a
+        // window stay candidates and tie at -inf with the other masked ones); all bounds fit an int.
         const int erows = (int)min((int64_t)128, d.E - e0);
-        const int vis0 = d.causal ? (int)max((int64_t)-4096, min((int64_t)4096, off + c0 - e0)) : 4096;
+        const int vis0 = block_vis0(d, c0, e0), win0 = block_win0(d, c0, e0);
         const int kk0 = (int)max((int64_t)-4096, (int64_t)kk - e0);
         const int64_t lane_at = (nb * d.C + c0 + 32 * wr + 4 * h) * d.E + e0 + 64 * wc + n32;
         const uint32_t off0 = 0xffffu - (uint32_t)(e0 - lo) - (uint32_t)(64 * wc + n32);
@@ -1191,7 +1221,7 @@ lmk_score_topk_fused_kernel(lmk_desc d, int kk, int nseg, int64_t seg_len, const
                     word = __float_as_uint(acc[t][r]);
                     half = (uint16_t)el;
                 } else if (rl < crows && el < cand_end) {
-                    const bool masked = !(el < vis);
+                    const bool masked = !(el < vis && el >= win0 + rl);
                     const float x = masked ? -INFINITY : finish_score<bf16_t>(acc[t][r], sqrt_hidden);
                     half = f_to_bf16_bits(x);
                     float sel = x;
@@ -1225,7 +1255,7 @@ lmk_score_topk_fused_kernel(lmk_desc d, int kk, int nseg, int64_t seg_len, const
                     key = ((uint64_t)word << 32) | cand_pay[i * 64 + rowl];
                 } else {
                     const int el = cand_pay[i * 64 + rowl];
-                    const bool masked = !(el < vis0 + rowl);
+                    const bool masked = !(el < vis0 + rowl && el >= win0 + rowl);
                     const float x = masked ? -INFINITY : finish_score<bf16_t>(__uint_as_float(word), sqrt_hidden);
                     key = (sortable_bits(x) & 0xffff0000u) | (0xffffu - (uint32_t)(e0 - lo) - (uint32_t)el);
                 }

@@ -17,6 +17,7 @@ GCA_F32, GCA_BF16 = 0, 1
 GCA_PATH_AUTO, GCA_PATH_GENERIC, GCA_PATH_MFMA = 0, 1, 2
 GCA_Q_HEAD_MAJOR, GCA_Q_TOKEN_MAJOR = 0, 1
 GCA_OK = 0
+GCA_ERR_SHAPE = 2
 
 SYMBOLS = (
     "gca_version", "gca_strerror", "gca_fwd", "gca_bwd_workspace_bytes", "gca_bwd", "gca_fwd_indexed",
@@ -42,12 +43,15 @@ class GcaDesc(ctypes.Structure):
     ]
 
 
+ABI_VERSION = 200       # gca_version() of the library whose structs these are (lmk_desc gained chunk_win in 200)
+
+
 class LmkDesc(ctypes.Structure):
     _fields_ = [
         ("dtype", ctypes.c_int32), ("topk", ctypes.c_int32),
         ("N", ctypes.c_int64), ("C", ctypes.c_int64), ("E", ctypes.c_int64),
         ("Dm", ctypes.c_int32), ("causal", ctypes.c_int32),
-        ("hidden_size", ctypes.c_float), ("lmk_k_rows", ctypes.c_int32),
+        ("hidden_size", ctypes.c_float), ("lmk_k_rows", ctypes.c_int32), ("chunk_win", ctypes.c_int32),
     ]
 
 
@@ -116,6 +120,10 @@ def lib():
                         "Run `make -C long-context-modeling_amd/csrc`.")
                 handle = ctypes.CDLL(LIB_PATH)
                 _declare(handle)
+                if handle.gca_version() != ABI_VERSION:      # the descriptors above must be the library's own
+                    raise RuntimeError(
+                        f"{LIB_PATH} is version {handle.gca_version()}, this package binds version {ABI_VERSION}: "
+                        "rebuild with `make -C long-context-modeling_amd/csrc`.")
                 _lib = handle
     return _lib
 

@@ -241,11 +241,14 @@ class ChunkKVManager:
                 self._cur_w[g] = self._cur_w[g].index_select(0, beam_idx.to(self._cur_w[g].device))
 
     # ---- the two retrieval sites of the model and the decode-step attention ----------------------------
-    def batch_retrieval(self, lmk_q, topk, group_idx=0, hidden_size=None, noise=None, use_cache=False):
+    def batch_retrieval(self, lmk_q, topk, group_idx=0, hidden_size=None, noise=None, use_cache=False,
+                        max_chunk_win=-1):
         """Scoring, mask, top-k and weights of ``lmk_q`` (N, C, Dl) against all stored landmarks
         (DRT._perform_batch_retrieval, DRT.py:609-641, without the gather).  With ``use_cache`` the last
-        row becomes the decode state of the group (DRT.py:638-639).  Returns (indices, weights) (N, C, kk)."""
-        _, indices, weights = landmark_retrieve(lmk_q, self.lmk_embs, topk, hidden_size, True, noise)
+        row becomes the decode state of the group (DRT.py:638-639).  ``max_chunk_win`` is the mask's window
+        (DRT.py:590-603; the model leaves it at -1).  Returns (indices, weights) (N, C, kk)."""
+        _, indices, weights = landmark_retrieve(lmk_q, self.lmk_embs, topk, hidden_size, True, noise, True,
+                                                max_chunk_win)
         if use_cache and not torch.is_grad_enabled():
             self.update_current_retrieved_chunk(indices, weights, group_idx)
         return indices, weights

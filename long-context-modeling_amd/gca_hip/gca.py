@@ -308,12 +308,12 @@ class _AttentionTokens(torch.autograd.Function):
         dq = torch.empty_like(q_tok)
         dq[:, 0].zero_()
         dkc, dvc = torch.empty_like(k_cache), torch.empty_like(v_cache)
-        dw = torch.zeros(w_shape, device=q_tok.device, dtype=torch.float32)      # last retrieval row: unused, gradient 0
+        dw = torch.zeros(w_shape, device=q_tok.device, dtype=w_dtype)            # last retrieval row: unused, gradient 0
         dwz = torch.empty((Z, kk), device=q_tok.device, dtype=torch.float32)
         desc = _desc(q_tok, kk, K_CTX, Dm // D, w, sm_scale, sm_n, N=Nc, C=Cc, token_shape=(Z, num_heads, S, D, 1))
         _bwd_indexed(desc, q_tok, k_cache, v_cache, idx, w, do, lse, dq, dkc, dvc, dwz, ctx.indices_src)
-        dw[:, :-1] = dwz.view(N, C - 1, kk)
-        return dq, dkc, dvc, None, dw.to(w_dtype), None, None, None, None
+        dw[:, :-1].copy_(dwz.view(N, C - 1, kk))                # rounds to the weights' type on the way
+        return dq, dkc, dvc, None, dw, None, None, None, None
 
 
 def attention_tokens(q_tok, k_cache, v_cache, indices, weights, num_heads, sm_n=0.0, sm_scale=None):

@@ -14,9 +14,27 @@ from . import _lib
 from .gca import _DT, _ptr, _stream
 
 
-def _lmk_desc(dtype, topk, N, C, E, Dm, causal, hidden_size, lmk_k_rows=0):
+def _lmk_desc(dtype, topk, N, C, E, Dm, causal, hidden_size, lmk_k_rows=0, max_chunk_win=-1):
+    """``max_chunk_win`` as in ``_enc_dec_score_mask`` (model/DRT.py:590-603): -1 no window, w >= 1 a row sees only
+    the w most recent chunks of its past.  (0 would hide everything; the callers below answer that case themselves.)"""
+    assert max_chunk_win == -1 or max_chunk_win >= 1
     return _lib.LmkDesc(dtype=_DT[dtype], topk=int(topk), N=N, C=C, E=E, Dm=Dm, causal=1 if causal else 0,
-                        hidden_size=float(hidden_size), lmk_k_rows=int(lmk_k_rows))
+                        hidden_size=float(hidden_size), lmk_k_rows=int(lmk_k_rows),
+                        chunk_win=0 if (max_chunk_win == -1 or not causal) else int(max_chunk_win))
+
+
+def _nothing_visible(causal, max_chunk_win):
+    """``max_chunk_win = 0`` under the causal mask: dec > enc and dec <= enc, no chunk is visible to any row."""
+    assert max_chunk_win >= -1
+    return bool(causal) and max_chunk_win == 0
+
+
+def _all_masked_selection(N, C, E, topk, device):
+    """What the kernels give for a row that sees nothing: the first kk chunks (every score ties at -inf, lower index
+    first) with weight 0 (softmax of -inf is NaN -> 0, model/DRT.py:626-627)."""
+    kk = min(E, int(topk))
+    indices = torch.arange(kk, device=device, dtype=torch.int64).expand(N, C, kk).contiguous()
+    return indices, torch.zeros((N, C, kk), device=device, dtype=torch.float32)
 
 
 def _dense_or_strided(lmk_k):
@@ -31,9 +49,9 @@ def _dense_or_strided(lmk_k):
     return lmk_k.contiguous(), 0
 
 
-def landmark_scores(lmk_q, lmk_k, hidden_size=None, causal=True):
-    """scores[n,c,e] = <lmk_q[n,c], lmk_k[n,e]> / sqrt(hidden), -inf where not strictly past
-    (model/DRT.py:612-613)."""
+def landmark_scores(lmk_q, lmk_k, hidden_size=None, causal=True, max_chunk_win=-1):
+    """scores[n,c,e] = <lmk_q[n,c], lmk_k[n,e]> / sqrt(hidden), -inf where not strictly past or, with
+    ``max_chunk_win`` = w, further back than w chunks (model/DRT.py:612-613, mask :590-607)."""
     assert lmk_q.is_cuda and lmk_q.dim() == 3 and lmk_k.dim() == 3 and lmk_q.dtype in _DT and lmk_k.dtype == lmk_q.dtype
     lmk_q = lmk_q.contiguous()
     lmk_k, rows = _dense_or_strided(lmk_k)
@@ -41,18 +59,21 @@ def landmark_scores(lmk_q, lmk_k, hidden_size=None, causal=True):
     E = lmk_k.shape[1]
     assert lmk_k.shape[0] == N and lmk_k.shape[2] == Dm
     hidden_size = Dm if hidden_size is None else hidden_size
+    if _nothing_visible(causal, max_chunk_win):
+        return torch.full((N, C, E), float("-inf"), device=lmk_q.device, dtype=lmk_q.dtype)
     scores = torch.empty((N, C, E), device=lmk_q.device, dtype=lmk_q.dtype)
-    desc = _lmk_desc(lmk_q.dtype, 1, N, C, E, Dm, causal, hidden_size, rows)
+    desc = _lmk_desc(lmk_q.dtype, 1, N, C, E, Dm, causal, hidden_size, rows, max_chunk_win)
     with torch.cuda.device(lmk_q.device):
         rc = _lib.lib().lmk_score(ctypes.byref(desc), _ptr(lmk_q), _ptr(lmk_k), _ptr(scores), _stream(lmk_q.device))
     _lib.check(rc, "lmk_score")
     return scores
 
 
-def landmark_topk(scores, topk, causal=True, noise=None):
+def landmark_topk(scores, topk, causal=True, noise=None, max_chunk_win=-1):
     """Top-k chunk ids and retrieval weights per row of ``scores`` (N, C, E)
     (model/DRT.py:613-627).  Returns (indices int64 (N,C,kk), weights float32 (N,C,kk)) with
-    kk = min(E, topk); order: higher (score+noise) first, ties by lower index."""
+    kk = min(E, topk); order: higher (score+noise) first, ties by lower index.  The mask (``causal``,
+    ``max_chunk_win``) is applied here as well."""
     assert scores.is_cuda and scores.dim() == 3 and scores.dtype in _DT
     scores = scores.contiguous()
     if noise is not None:
@@ -60,9 +81,11 @@ def landmark_topk(scores, topk, causal=True, noise=None):
         noise = noise.contiguous()
     N, C, E = scores.shape
     kk = min(E, int(topk))
+    if _nothing_visible(causal, max_chunk_win):
+        return _all_masked_selection(N, C, E, topk, scores.device)
     indices = torch.empty((N, C, kk), device=scores.device, dtype=torch.int64)
     weights = torch.empty((N, C, kk), device=scores.device, dtype=torch.float32)
-    desc = _lmk_desc(scores.dtype, topk, N, C, E, 1, causal, 1.0)
+    desc = _lmk_desc(scores.dtype, topk, N, C, E, 1, causal, 1.0, 0, max_chunk_win)
     with torch.cuda.device(scores.device):
         L = _lib.lib()
         nbytes = L.lmk_topk_workspace_bytes(ctypes.byref(desc))
@@ -77,7 +100,7 @@ FUSED_MIN_BYTES = 2 << 30
 
 
 def landmark_score_topk(lmk_q, lmk_k, topk, hidden_size=None, causal=True, noise=None, return_scores=True,
-                        fused=None):
+                        fused=None, max_chunk_win=-1):
     """Scoring and selection through the one-call entry point ``lmk_score_topk`` (model/DRT.py:612-627).
     Returns (scores or None, indices, weights).  With ``return_scores=False`` and a score matrix of at least
     ``FUSED_MIN_BYTES`` (2 GiB) the matrix is never written: the fused kernel (bf16, width a multiple of 64, at
@@ -99,13 +122,13 @@ def landmark_score_topk(lmk_q, lmk_k, topk, hidden_size=None, causal=True, noise
     dev = lmk_q.device
     if fused is None:
         fused = N * C * E * lmk_q.element_size() >= FUSED_MIN_BYTES
-    if return_scores or not fused:
-        scores = landmark_scores(lmk_q, lmk_k, hidden_size, causal)
-        indices, weights = landmark_topk(scores, topk, causal, noise)
+    if return_scores or not fused or _nothing_visible(causal, max_chunk_win):
+        scores = landmark_scores(lmk_q, lmk_k, hidden_size, causal, max_chunk_win)
+        indices, weights = landmark_topk(scores, topk, causal, noise, max_chunk_win)
         return (scores if return_scores else None), indices, weights
     indices = torch.empty((N, C, kk), device=dev, dtype=torch.int64)
     weights = torch.empty((N, C, kk), device=dev, dtype=torch.float32)
-    desc = _lmk_desc(lmk_q.dtype, topk, N, C, E, Dm, causal, hidden_size, rows)
+    desc = _lmk_desc(lmk_q.dtype, topk, N, C, E, Dm, causal, hidden_size, rows, max_chunk_win)
     with torch.cuda.device(dev):
         L = _lib.lib()
         nbytes = L.lmk_topk_workspace_bytes(ctypes.byref(desc))
@@ -113,8 +136,8 @@ def landmark_score_topk(lmk_q, lmk_k, topk, hidden_size=None, causal=True, noise
         rc = L.lmk_score_topk(ctypes.byref(desc), _ptr(lmk_q), _ptr(lmk_k), _ptr(noise), None, _ptr(indices),
                               _ptr(weights), _ptr(ws), nbytes, _stream(dev))
     if rc == _lib.GCA_ERR_UNSUPPORTED:
-        full = landmark_scores(lmk_q, lmk_k, hidden_size, causal)
-        indices, weights = landmark_topk(full, topk, causal, noise)
+        full = landmark_scores(lmk_q, lmk_k, hidden_size, causal, max_chunk_win)
+        indices, weights = landmark_topk(full, topk, causal, noise, max_chunk_win)
         return None, indices, weights
     _lib.check(rc, "lmk_score_topk")
     return None, indices, weights
@@ -125,9 +148,10 @@ class _Retrieve(torch.autograd.Function):
     embeddings (what autograd does through model/DRT.py:612 and :626-627); the selection is constant."""
 
     @staticmethod
-    def forward(ctx, lmk_q, lmk_k, topk, hidden_size, causal, noise, return_scores):
+    def forward(ctx, lmk_q, lmk_k, topk, hidden_size, causal, noise, return_scores, max_chunk_win):
         lmk_q, lmk_k = lmk_q.contiguous(), lmk_k.contiguous()
-        scores, indices, weights = landmark_score_topk(lmk_q, lmk_k, topk, hidden_size, causal, noise, return_scores)
+        scores, indices, weights = landmark_score_topk(lmk_q, lmk_k, topk, hidden_size, causal, noise, return_scores,
+                                                       None, max_chunk_win)
         ctx.save_for_backward(lmk_q, lmk_k, indices, weights)
         ctx.hidden, ctx.topk, ctx.causal = float(hidden_size), int(topk), bool(causal)
         if scores is None:
@@ -150,19 +174,22 @@ class _Retrieve(torch.autograd.Function):
             rc = L.lmk_weights_bwd(ctypes.byref(desc), _ptr(lmk_q), _ptr(lmk_k), _ptr(indices), _ptr(weights),
                                    _ptr(dweights), _ptr(dlq), _ptr(dlk), _ptr(ws), nbytes, _stream(lmk_q.device))
         _lib.check(rc, "lmk_weights_bwd")
-        return dlq, dlk, None, None, None, None, None
+        return dlq, dlk, None, None, None, None, None, None
 
 
-def landmark_retrieve(lmk_q, lmk_k, topk, hidden_size=None, causal=True, noise=None, return_scores=True):
+def landmark_retrieve(lmk_q, lmk_k, topk, hidden_size=None, causal=True, noise=None, return_scores=True,
+                      max_chunk_win=-1):
     """Scoring + selection in one call.  Returns (scores, indices, weights); ``weights`` carries the
     gradient to ``lmk_q`` and ``lmk_k``.  ``return_scores=False`` returns None for the scores and lets the fused
-    kernel skip the (N, C, E) matrix (see ``landmark_score_topk``)."""
+    kernel skip the (N, C, E) matrix (see ``landmark_score_topk``).  ``max_chunk_win`` is the window of
+    ``_enc_dec_score_mask`` (model/DRT.py:590-603): -1 none, w a row sees its w most recent past chunks only."""
     assert lmk_q.is_cuda and lmk_q.dim() == 3 and lmk_k.dim() == 3
     hidden_size = lmk_q.shape[-1] if hidden_size is None else hidden_size
     if not (torch.is_grad_enabled() and (lmk_q.requires_grad or lmk_k.requires_grad)):
         # inference: no copy of a landmark store that is a view with spare capacity
-        return landmark_score_topk(lmk_q, lmk_k, topk, hidden_size, causal, noise, return_scores)
-    scores, indices, weights = _Retrieve.apply(lmk_q, lmk_k, topk, hidden_size, causal, noise, return_scores)
+        return landmark_score_topk(lmk_q, lmk_k, topk, hidden_size, causal, noise, return_scores, None, max_chunk_win)
+    scores, indices, weights = _Retrieve.apply(lmk_q, lmk_k, topk, hidden_size, causal, noise, return_scores,
+                                               max_chunk_win)
     return (scores if return_scores else None), indices, weights
 
 

@@ -30,7 +30,8 @@ def test_struct_layout_matches_header():
     # offsets implied by the C declaration order with natural alignment
     assert ctypes.sizeof(_lib.GcaDesc) == 80 and _lib.GcaDesc.Z.offset == 8 and _lib.GcaDesc.N.offset == 56
     assert _lib.GcaDesc.q_layout.offset == 72 and _lib.GcaDesc.q_skip.offset == 76
-    assert ctypes.sizeof(_lib.LmkDesc) == 48 and _lib.LmkDesc.E.offset == 24 and _lib.LmkDesc.hidden_size.offset == 40
+    assert ctypes.sizeof(_lib.LmkDesc) == 56 and _lib.LmkDesc.E.offset == 24 and _lib.LmkDesc.hidden_size.offset == 40
+    assert _lib.LmkDesc.lmk_k_rows.offset == 44 and _lib.LmkDesc.chunk_win.offset == 48
 
 
 def _desc(**kw):
@@ -42,7 +43,7 @@ def _desc(**kw):
 
 def test_validation_without_gpu():
     L = _lib.lib()
-    assert L.gca_version() >= 100
+    assert L.gca_version() >= 200
     one = ctypes.c_void_p(16)   # never dereferenced: validation fails first
     null = ctypes.c_void_p(0)
     assert L.gca_fwd(None, one, one, one, one, one, null, null) == 1
