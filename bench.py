@@ -209,7 +209,8 @@ def run_cfg2_gathered(torch, dev, seed, iters):
     gemm = 2 * Z * H * K * S * S * d
     e = 2
     q_b, g_b, lse_b = Z * H * S * d * e, Z * H * K * S * d * e, Z * H * K * S * 4
-    nbytes = (2 * q_b + 2 * g_b + lse_b) + (3 * q_b + 2 * g_b + 2 * lse_b) + (2 * q_b + 4 * g_b + 2 * lse_b)
+    # forward: q, o, K, V, lse; backward (one launch): q, dO, dq, K, V, dk, dv, lse, delta
+    nbytes = (2 * q_b + 2 * g_b + lse_b) + (3 * q_b + 4 * g_b + 2 * lse_b)
     out = {"tokens_per_s": round(tokens / t, 1), "ms": round(t * 1e3, 4)}
     out.update(bound_of(7 * gemm, nbytes, t))
     out["with_reference_style_gather_and_scatter"] = {"tokens_per_s": round(tokens / t2, 1), "ms": round(t2 * 1e3, 4)}

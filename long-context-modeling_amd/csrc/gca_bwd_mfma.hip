@@ -216,6 +216,252 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
         }
 }
 
+// ------------------------------------------------------------------------------- gathered form, one launch
+//
+// With gathered K/V every query chunk has its own copy of its K retrieved chunks, so dk / dv of slot (z, kv head, j)
+// receive nothing from any other query chunk: when the kv head has one query head and the chunk one 64-row query
+// tile, the dq kernel's workgroup already sees everything that goes into them.  This kernel is the dq kernel for that
+// case with the two remaining products added, five products per (head, chunk) instead of seven and K / V read
+// from HBM once instead of twice:
+//      P~ (= |w| sm_scale P) and dS, rounded to bf16, go to LDS as [query][key] tiles (8-byte writes of the
+//      registers as they are); after a barrier wavefront kb reads the columns of key block kb back transposed
+//      (ds_read_tr16_b64: lane = key, reduction slots = queries) and forms
+//      dV^T = dO^T P~,  dK^T = Q^T dS      dO^T / Q^T (lane = dim, slots = queries) are read once per workgroup
+//                                          the same way and stay in registers
+//      so every lane ends up with its key row's dims in its registers, as the dq accumulators hold a query row's.
+// dV is rescaled by sign(w) / sm_scale on the way out.  A slot of weight 0 writes zeros.
+template <int D>
+__global__ void __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2)))
+gca_bwd_gathered_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
+                             const uint16_t* __restrict__ v, const void* __restrict__ w, int w_is_bf16,
+                             const uint16_t* __restrict__ dout, const float* __restrict__ lse,
+                             uint16_t* __restrict__ dq, uint16_t* __restrict__ dk, uint16_t* __restrict__ dv,
+                             float* __restrict__ delta) {
+    static_assert(D == 64, "register budget of the stationary transposed operands");
+    constexpr int NT = 128;
+    constexpr int KS = D / 16, DB = D / 32;
+    constexpr int RB = D * 2, TILE = 64 * RB;
+    // two K tiles, one V tile, the P~ and dS exchange tiles (which first hold Q and dO)
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[5 * TILE];
+    unsigned char* const xP = smem + 3 * TILE;
+    unsigned char* const xS = smem + 4 * TILE;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 31, h = lane >> 5;
+    int64_t bid = xcd_logical(blockIdx.x, p.Z * p.Hkv);
+    if (bid < 0) return;
+    const int64_t z = bid % p.Z;
+    const int hk = (int)(bid / p.Z);          // one query head per kv head: hq == hk
+    const int q0 = wave * 32;
+    const int qrs = (int)p.q_rs;
+    const int64_t qoff = q_base_n(p, 0, z, hk);
+
+    const TileLoader<D, NT> loader(tid, D);
+    {
+        const TileLoader<D, NT> qloader(tid, qrs);
+        qloader.issue(q + qoff, xP);
+        qloader.issue(dout + qoff, xS);
+        int64_t rs;
+        loader.issue(chunk_base_n(p, k, nullptr, 0, z, hk, 0, rs), smem);
+        loader.issue(chunk_base_n(p, v, nullptr, 0, z, hk, 0, rs), smem + 2 * TILE);
+    }
+    bf16x8 qB[KS], doB[KS];
+    {
+        const int64_t off = qoff + (q0 + n) * qrs + 8 * h;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            qB[ks] = *reinterpret_cast<const bf16x8*>(q + off + 16 * ks);
+            doB[ks] = *reinterpret_cast<const bf16x8*>(dout + off + 16 * ks);
+        }
+    }
+    f32x16 dqacc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dqacc[db][r] = 0.f;
+
+    const float c = p.sm_scale * LOG2E;
+    const TrLane tr(lane);
+    const int fsw = swz(n);
+    const int64_t lrow = (z * p.Hq + hk) * (int64_t)p.K * p.Q_CTX + q0 + n;
+
+    wait_async_tiles();
+    __syncthreads();
+    // Q^T and dO^T as A operands: lane = dim 32*db + n, slots = the 16 queries of step t4
+    bf16x8 qT[4][DB], doT[4][DB];
+#pragma unroll
+    for (int t4 = 0; t4 < 4; ++t4)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            const int o0 = tr.off(t4, db, RB);
+            qT[t4][db] = lds_read_tr_pair(xP + o0, xP + o0 + 8 * RB);
+            doT[t4][db] = lds_read_tr_pair(xS + o0, xS + o0 + 8 * RB);
+        }
+    // (the exchange tiles are first written after the barrier in the middle of chunk 0, which every wavefront
+    // reaches with these reads behind it)
+
+    // this lane's 8-byte pieces of its query row in an exchange tile: keys 32t + 8a + 4h .. + 3
+    const int xrow = (q0 + n) * RB + 8 * h;
+    float lse_next = lse[lrow];
+    for (int j = 0; j < p.K; ++j) {
+        const int buf = j & 1;
+        const bool more = j + 1 < p.K;
+        const float lse_cur = lse_next;
+        if (more) {
+            lse_next = lse[lrow + (int64_t)(j + 1) * p.Q_CTX];
+            int64_t rs;
+            loader.issue(chunk_base_n(p, k, nullptr, 0, z, hk, j + 1, rs), smem + (buf ^ 1) * TILE);
+        }
+        const float wj = load_w(w, w_is_bf16, z * p.K + j);
+        const float mult = wj * p.sm_scale;
+        const float amult = fabsf(mult);
+        const bool live = amult > 0.f;
+        const float eoff = lse_cur - (live ? __builtin_amdgcn_logf(amult) : 0.f);
+        const float dscale = live ? 1.f / amult : 1.f;
+        const unsigned char* kb = smem + buf * TILE;
+        const unsigned char* vb = smem + 2 * TILE;
+
+        f32x16 st[2], dpt[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { st[t][r] = 0.f; dpt[t][r] = 0.f; }
+            const int rowoff = (32 * t + n) * RB;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int po = rowoff + (((2 * ks + h) ^ fsw) << 4);
+                st[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(kb + po), qB[ks], st[t], 0, 0, 0);
+                dpt[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(vb + po), doB[ks], dpt[t], 0, 0, 0);
+            }
+        }
+        // every wavefront is done with the V tile, and with the previous chunk's exchange tiles
+        __syncthreads();
+        if (more) {
+            int64_t rs;
+            loader.issue(chunk_base_n(p, v, nullptr, 0, z, hk, j + 1, rs), smem + 2 * TILE);
+        }
+        float dsum = 0.f;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float pe = __builtin_amdgcn_exp2f(fmaf(st[t][r], c, -eoff));
+                st[t][r] = pe;
+                dsum = fmaf(pe, dpt[t][r], dsum);
+            }
+        dsum += __shfl_xor(dsum, 32);
+        dsum *= dscale;                                   // D_j = rowsum(P * dP)
+        if (h == 0) delta[lrow + (int64_t)j * p.Q_CTX] = dsum;
+
+        f32x16 dvacc[DB], dkacc[DB];
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { dvacc[db][r] = 0.f; dkacc[db][r] = 0.f; }
+
+        if (live) {                                       // uniform over the workgroup: one weight per (z, j)
+            bf16x8 dsA[4], pA[4];
+#pragma unroll
+            for (int t4 = 0; t4 < 4; ++t4)
+#pragma unroll
+                for (int s = 0; s < 8; ++s) {
+                    const int r = 8 * (t4 & 1) + s;
+                    dsA[t4][s] = (__bf16)(st[t4 >> 1][r] * (dpt[t4 >> 1][r] - dsum));
+                    pA[t4][s] = (__bf16)st[t4 >> 1][r];
+                }
+            if (mult < 0.f) {
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int t4 = 0; t4 < 4; ++t4) dsA[t4] = negate_bf16x8(dsA[t4]);
+            }
+            // registers 8*(t4&1) + 4*(a&1) + e of tile t = t4/2 are keys 32t + 8a + 4h + e, a = 2*(t4&1) + ..: piece 4t + a
+#pragma unroll
+            for (int t4 = 0; t4 < 4; ++t4)
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int piece = 4 * (t4 >> 1) + 2 * (t4 & 1) + half;
+                    const int off = xrow + ((piece ^ fsw) << 4);
+                    union { bf16x8 v; uint64_t u[2]; } a, b;
+                    a.v = pA[t4];
+                    b.v = dsA[t4];
+                    *reinterpret_cast<uint64_t*>(xP + off) = a.u[half];
+                    *reinterpret_cast<uint64_t*>(xS + off) = b.u[half];
+                }
+#pragma unroll
+            for (int t4 = 0; t4 < 4; ++t4)
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    const int o0 = tr.off(t4, db, RB);
+                    const bf16x8 b = lds_read_tr_pair(kb + o0, kb + o0 + 8 * RB);
+                    dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, dsA[t4], dqacc[db], 0, 0, 0);
+                }
+            __syncthreads();
+            // key block `wave`: lane = key 32*wave + n, slots = the 16 queries of step t4
+#pragma unroll
+            for (int t4 = 0; t4 < 4; ++t4) {
+                const int o0 = tr.off(t4, wave, RB);
+                const bf16x8 pT = lds_read_tr_pair(xP + o0, xP + o0 + 8 * RB);
+                const bf16x8 sT = lds_read_tr_pair(xS + o0, xS + o0 + 8 * RB);
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(doT[t4][db], pT, dvacc[db], 0, 0, 0);
+                    dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qT[t4][db], sT, dkacc[db], 0, 0, 0);
+                }
+            }
+        }
+
+        wait_async_tiles();
+        __syncthreads();
+
+        // dk / dv of slot j.  The accumulators hold the lane's key row, registers 4a .. 4a+3 of block db being dims
+        // 32*db + 8a + 4h + 0..3; stored like that, an instruction would touch 32 rows with 16 bytes each.  The
+        // wavefront's 32 rows go through its own rows of the exchange tiles instead (free until the next chunk's
+        // exchange, and no other wavefront touches them before the next barrier) and leave as 16-byte pieces, eight
+        // lanes to a 128-byte row: 1 KB contiguous per instruction.  Issued after the wait above, so the stores are
+        // long done when the next chunk's wait comes.
+        {
+            const float vscale = live ? (mult < 0.f ? -1.f : 1.f) / p.sm_scale : 0.f;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    union { __bf16 b[4]; uint64_t u; } pk, pv;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        pk.b[e] = (__bf16)dkacc[db][4 * a + e];
+                        pv.b[e] = (__bf16)(dvacc[db][4 * a + e] * vscale);
+                    }
+                    const int off = xrow + (((4 * db + a) ^ fsw) << 4);
+                    *reinterpret_cast<uint64_t*>(xP + off) = pk.u;
+                    *reinterpret_cast<uint64_t*>(xS + off) = pv.u;
+                }
+            int64_t rs;
+            const int64_t slot = chunk_base_n(p, k, nullptr, 0, z, hk, j, rs) - k;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = 32 * wave + 8 * i + (lane >> 3), lp = lane & 7;
+                const int off = tile_off(row, lp, RB);
+                const u32x4 kq = *reinterpret_cast<const u32x4*>(xP + off);
+                const u32x4 vq = *reinterpret_cast<const u32x4*>(xS + off);
+                *reinterpret_cast<u32x4*>(dk + slot + row * D + lp * 8) = kq;
+                *reinterpret_cast<u32x4*>(dv + slot + row * D + lp * 8) = vq;
+            }
+        }
+    }
+
+    uint16_t* dqp = dq + qoff + (int64_t)(q0 + n) * qrs + 4 * h;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            union { __bf16 b[4]; uint64_t u; } pk;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pk.b[e] = (__bf16)dqacc[db][4 * a + e];
+            *reinterpret_cast<uint64_t*>(dqp + 32 * db + 8 * a) = pk.u;
+        }
+}
+
 // ------------------------------------------------------------------------------------------- dkdv
 
 // Two-wavefront variant of the dk/dv kernel, used for D == 64: each wavefront owns 32 key rows and does
@@ -804,6 +1050,19 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
                         int wb, const void* dout, const float* lse, void* dq, void* dk, void* dv, float* dw,
                         float* delta, void* lists, hipStream_t s) {
     int rc = GCA_OK;
+    if constexpr (D == 64) {
+        // gathered form, one query head per kv head, one query tile: dq, dk and dv in one launch
+        const int both = GCA_STAGE_DQ | GCA_STAGE_DKDV;
+        if (!p.indexed && p.G == 1 && p.Q_CTX == 64 && (p.stages & both) == both) {
+            const int64_t blocks = xcd_grid(p.Z * p.Hkv);
+            if (blocks <= 0 || blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
+            hipLaunchKernelGGL((gca_bwd_gathered_mfma_kernel<D>), dim3((unsigned)blocks), dim3(128), 0, s, p,
+                               (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
+                               (uint16_t*)dq, (uint16_t*)dk, (uint16_t*)dv, delta);
+            if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
+            return (p.stages & GCA_STAGE_DW) ? launch_dw(p, delta, dw, s) : GCA_OK;
+        }
+    }
     if (p.stages & GCA_STAGE_DQ) {
         // d=128: two heads per workgroup (4 wavefronts, two workgroups per CU at 234 VGPRs) instead of four, as in the
         // forward: independent workgroups overlap their phases (3.80 against 3.89 ms at B=4 Hq=32 Hkv=8 L=32K k=16)
