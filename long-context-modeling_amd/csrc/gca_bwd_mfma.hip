@@ -1,7 +1,7 @@
 // GCA backward on the gfx950 matrix cores (bf16 in, fp32 accumulate).  Same shape class as the
 // MFMA forward: bf16, K_CTX == 64, D in {64, 128}, Q_CTX % 64 == 0, sm_scale > 0.
 //
-// Two kernels, five + two products per (query head, retrieved chunk):
+// Two kernels, five + two products per (query head, retrieved chunk), and a one-launch form for gathered K/V:
 //
 // 1. dq kernel -- query-centric, the forward's work split (workgroup = (z, kv head, GS query heads,
 //    64 query rows), wavefront = 32 query rows, K/V tiles of the retrieved chunks double-buffered in LDS).
@@ -27,6 +27,8 @@
 //    order is fixed); dk/dv come out in bf16 in the cache's own layout, every element written once.
 //    Lists longer than SEG_MAX are cut into segments handled by separate workgroups that write float
 //    partial tiles; a small reduce launch adds those up in segment order.
+//
+// 3. gathered form with one query head per kv head (d = 64): kernel 1 with dk / dv added, one launch (see there).
 //
 // dw[z, j] = sum over heads and rows of delta (shared launch_dw).
 #include "gca_mfma.h"
