@@ -215,3 +215,22 @@ def test_validation_of_the_list_fused_and_static_entry_points():
     assert L.lmk_score_topk_static(ctypes.byref(too_big), one, one, null, one, one, null) == _lib.GCA_ERR_SCRATCH_LIMIT
     assert L.lmk_score_topk_static(ctypes.byref(too_big), null, one, null, one, one, null) == 1
     assert b"scratch" in L.gca_strerror(_lib.GCA_ERR_SCRATCH_LIMIT).lower()
+
+
+def test_chunk_window_of_the_landmark_descriptor():
+    """``max_chunk_win`` of the mask (model/DRT.py:590-603) maps to ``lmk_desc.chunk_win`` (0 = none); a negative
+    field is refused before anything touches a GPU."""
+    import torch
+    from gca_hip.retrieval import _lmk_desc, _nothing_visible
+    assert _lmk_desc(torch.bfloat16, 8, 1, 64, 64, 64, True, 64.0).chunk_win == 0
+    assert _lmk_desc(torch.bfloat16, 8, 1, 64, 64, 64, True, 64.0, 0, -1).chunk_win == 0
+    assert _lmk_desc(torch.bfloat16, 8, 1, 64, 64, 64, True, 64.0, 0, 5).chunk_win == 5
+    assert _lmk_desc(torch.bfloat16, 8, 1, 64, 64, 64, False, 64.0, 0, 5).chunk_win == 0      # no mask, no window
+    assert _nothing_visible(True, 0) and not _nothing_visible(False, 0) and not _nothing_visible(True, 3)
+    with pytest.raises(AssertionError):
+        _lmk_desc(torch.bfloat16, 8, 1, 64, 64, 64, True, 64.0, 0, 0)
+    L = _lib.lib()
+    one = ctypes.c_void_p(16)
+    bad = _lib.LmkDesc(dtype=1, topk=8, N=1, C=64, E=64, Dm=64, causal=1, hidden_size=64.0, chunk_win=-2)
+    assert L.lmk_score(ctypes.byref(bad), one, one, one, None) == _lib.GCA_ERR_SHAPE
+    assert L.lmk_topk_workspace_bytes(ctypes.byref(bad)) == 0
