@@ -221,49 +221,67 @@ gca_bwd_dq_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t*
 // ------------------------------------------------------------------------------- gathered form, one launch
 //
 // With gathered K/V every query chunk has its own copy of its K retrieved chunks, so dk / dv of slot (z, kv head, j)
-// receive nothing from any other query chunk: when the kv head has one query head and the chunk one 64-row query
-// tile, the dq kernel's workgroup already sees everything that goes into them.  This kernel is the dq kernel for that
-// case with the two remaining products added, five products per (head, chunk) instead of seven and K / V read
-// from HBM once instead of twice:
-//      P~ (= |w| sm_scale P) and dS, rounded to bf16, go to LDS as [query][key] tiles (8-byte writes of the
-//      registers as they are); after a barrier wavefront kb reads the columns of key block kb back transposed
-//      (ds_read_tr16_b64: lane = key, reduction slots = queries) and forms
-//      dV^T = dO^T P~,  dK^T = Q^T dS      dO^T / Q^T (lane = dim, slots = queries) are read once per workgroup
-//                                          the same way and stay in registers
-//      so every lane ends up with its key row's dims in its registers, as the dq accumulators hold a query row's.
+// receive nothing from any other query chunk: a workgroup that holds all G query heads of the kv head and the
+// chunk's one 64-row query tile sees everything that goes into them.  This kernel is the dq kernel for that case
+// (workgroup = (z, kv head), 2 G wavefronts: wavefront (gs, qb) owns 32 query rows of head gs) with the two
+// remaining products added -- five products per (head, chunk) instead of seven, K / V read from HBM once
+// instead of twice:
+//      P~ (= |w| sm_scale P) and dS, rounded to bf16, go to LDS as [query][key] tiles of 64 G rows (8-byte writes
+//      of the registers as they are); after a barrier they are read back transposed (ds_read_tr16_b64: lane = key,
+//      reduction slots = queries) and every wavefront forms its share of
+//      dV^T = dO^T P~,  dK^T = Q^T dS      (2 tensors x 2 key blocks x 2 dim blocks of 32 x 32, reduction over the
+//                                          64 G query rows, dealt over the 2 G wavefronts)
+//      with its rows of dO^T / Q^T (lane = dim, slots = queries) read once per workgroup the same way and kept in
+//      registers.  Every lane ends up with its key row's dims in its registers, as the dq accumulators hold a
+//      query row's.
 // dV is rescaled by sign(w) / sm_scale on the way out.  A slot of weight 0 writes zeros.
-template <int D>
-__global__ void __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2)))
+template <int D, int G>
+__global__ void __launch_bounds__(128 * G) __attribute__((amdgpu_waves_per_eu(2)))
 gca_bwd_gathered_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
                              const uint16_t* __restrict__ v, const void* __restrict__ w, int w_is_bf16,
                              const uint16_t* __restrict__ dout, const float* __restrict__ lse,
                              uint16_t* __restrict__ dq, uint16_t* __restrict__ dk, uint16_t* __restrict__ dv,
                              float* __restrict__ delta) {
     static_assert(D == 64, "register budget of the stationary transposed operands");
-    constexpr int NT = 128;
+    static_assert(G == 1 || G == 2 || G == 4, "eight 32 x 32 output blocks are dealt over 2 G wavefronts");
+    constexpr int NT = 128 * G;
     constexpr int KS = D / 16, DB = D / 32;
     constexpr int RB = D * 2, TILE = 64 * RB;
-    // two K tiles, one V tile, the P~ and dS exchange tiles (which first hold Q and dO)
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[5 * TILE];
+    constexpr int XT = G * TILE;                 // an exchange tile: 64 G query rows x 64 keys
+    constexpr int T = 4 * G;                     // 16-query reduction steps of dk / dv
+    constexpr int NTEN = G == 1 ? 2 : 1;         // tensors (dk, dv) per wavefront
+    constexpr int NDB = G == 4 ? 1 : 2;          // 32-dim blocks per wavefront
+    // two K tiles, one V tile, the P~ and dS exchange tiles (which first hold Q and dO of the G heads)
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[3 * TILE + 2 * XT];
     unsigned char* const xP = smem + 3 * TILE;
-    unsigned char* const xS = smem + 4 * TILE;
+    unsigned char* const xS = xP + XT;
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31, h = lane >> 5;
+    const int gs = wave >> 1, qb = wave & 1;
     int64_t bid = xcd_logical(blockIdx.x, p.Z * p.Hkv);
     if (bid < 0) return;
     const int64_t z = bid % p.Z;
-    const int hk = (int)(bid / p.Z);          // one query head per kv head: hq == hk
-    const int q0 = wave * 32;
+    const int hk = (int)(bid / p.Z);
+    const int hq = hk * G + gs;
+    const int q0 = qb * 32;
     const int qrs = (int)p.q_rs;
-    const int64_t qoff = q_base_n(p, 0, z, hk);
+    const int64_t qoff = q_base_n(p, 0, z, hq);
+    // this wavefront's share of dk / dv: key block kb, tensors ten0 .. (0 = dk, 1 = dv), dim blocks db0 ..
+    const int kb = G == 1 ? wave : (G == 2 ? (wave & 1) : ((wave >> 1) & 1));
+    const int ten0 = G == 1 ? 0 : (G == 2 ? (wave >> 1) : (wave >> 2));
+    const int db0 = G == 4 ? (wave & 1) : 0;
 
     const TileLoader<D, NT> loader(tid, D);
     {
         const TileLoader<D, NT> qloader(tid, qrs);
-        qloader.issue(q + qoff, xP);
-        qloader.issue(dout + qoff, xS);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const int64_t o = q_base_n(p, 0, z, hk * G + g);
+            qloader.issue(q + o, xP + g * TILE);
+            qloader.issue(dout + o, xS + g * TILE);
+        }
         int64_t rs;
         loader.issue(chunk_base_n(p, k, nullptr, 0, z, hk, 0, rs), smem);
         loader.issue(chunk_base_n(p, v, nullptr, 0, z, hk, 0, rs), smem + 2 * TILE);
@@ -286,25 +304,31 @@ gca_bwd_gathered_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uin
     const float c = p.sm_scale * LOG2E;
     const TrLane tr(lane);
     const int fsw = swz(n);
-    const int64_t lrow = (z * p.Hq + hk) * (int64_t)p.K * p.Q_CTX + q0 + n;
+    const int64_t lrow = (z * p.Hq + hq) * (int64_t)p.K * p.Q_CTX + q0 + n;
 
     wait_async_tiles();
     __syncthreads();
-    // Q^T and dO^T as A operands: lane = dim 32*db + n, slots = the 16 queries of step t4
-    bf16x8 qT[4][DB], doT[4][DB];
+    // Q^T (for dk) / dO^T (for dv) as A operands: lane = dim 32*db + n, slots = the 16 queries of step t
+    bf16x8 aT[NTEN][T][NDB];
 #pragma unroll
-    for (int t4 = 0; t4 < 4; ++t4)
+    for (int ti = 0; ti < NTEN; ++ti) {
+        const unsigned char* src = (ten0 + ti) == 0 ? xP : xS;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-            const int o0 = tr.off(t4, db, RB);
-            qT[t4][db] = lds_read_tr_pair(xP + o0, xP + o0 + 8 * RB);
-            doT[t4][db] = lds_read_tr_pair(xS + o0, xS + o0 + 8 * RB);
-        }
+        for (int t = 0; t < T; ++t)
+#pragma unroll
+            for (int di = 0; di < NDB; ++di) {
+                const int o0 = tr.off(t, db0 + di, RB);
+                aT[ti][t][di] = lds_read_tr_pair(src + o0, src + o0 + 8 * RB);
+            }
+    }
     // (the exchange tiles are first written after the barrier in the middle of chunk 0, which every wavefront
     // reaches with these reads behind it)
 
     // this lane's 8-byte pieces of its query row in an exchange tile: keys 32t + 8a + 4h .. + 3
-    const int xrow = (q0 + n) * RB + 8 * h;
+    const int xrow = (gs * 64 + q0 + n) * RB + 8 * h;
+    // and of its key row where dk / dv are staged for the stores
+    const int krow = (32 * kb + n) * RB + 8 * h;
+
     float lse_next = lse[lrow];
     for (int j = 0; j < p.K; ++j) {
         const int buf = j & 1;
@@ -321,8 +345,8 @@ gca_bwd_gathered_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uin
         const bool live = amult > 0.f;
         const float eoff = lse_cur - (live ? __builtin_amdgcn_logf(amult) : 0.f);
         const float dscale = live ? 1.f / amult : 1.f;
-        const unsigned char* kb = smem + buf * TILE;
-        const unsigned char* vb = smem + 2 * TILE;
+        const unsigned char* kbuf = smem + buf * TILE;
+        const unsigned char* vbuf = smem + 2 * TILE;
 
         f32x16 st[2], dpt[2];
 #pragma unroll
@@ -333,11 +357,11 @@ gca_bwd_gathered_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uin
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 const int po = rowoff + (((2 * ks + h) ^ fsw) << 4);
-                st[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(kb + po), qB[ks], st[t], 0, 0, 0);
-                dpt[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(vb + po), doB[ks], dpt[t], 0, 0, 0);
+                st[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(kbuf + po), qB[ks], st[t], 0, 0, 0);
+                dpt[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_read_b128(vbuf + po), doB[ks], dpt[t], 0, 0, 0);
             }
         }
-        // every wavefront is done with the V tile, and with the previous chunk's exchange tiles
+        // every wavefront is done with the V tile, and with the previous chunk's exchange and staging areas
         __syncthreads();
         if (more) {
             int64_t rs;
@@ -356,11 +380,13 @@ gca_bwd_gathered_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uin
         dsum *= dscale;                                   // D_j = rowsum(P * dP)
         if (h == 0) delta[lrow + (int64_t)j * p.Q_CTX] = dsum;
 
-        f32x16 dvacc[DB], dkacc[DB];
+        f32x16 acc[NTEN][NDB];
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
+        for (int ti = 0; ti < NTEN; ++ti)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) { dvacc[db][r] = 0.f; dkacc[db][r] = 0.f; }
+            for (int di = 0; di < NDB; ++di)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[ti][di][r] = 0.f;
 
         if (live) {                                       // uniform over the workgroup: one weight per (z, j)
             bf16x8 dsA[4], pA[4];
@@ -377,7 +403,7 @@ gca_bwd_gathered_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uin
 #pragma unroll
                 for (int t4 = 0; t4 < 4; ++t4) dsA[t4] = negate_bf16x8(dsA[t4]);
             }
-            // registers 8*(t4&1) + 4*(a&1) + e of tile t = t4/2 are keys 32t + 8a + 4h + e, a = 2*(t4&1) + ..: piece 4t + a
+            // registers 8*(t4&1) + 4*half + e of key tile t4/2 are keys 32*(t4/2) + 8a + 4h + e, a = 2*(t4&1) + half
 #pragma unroll
             for (int t4 = 0; t4 < 4; ++t4)
 #pragma unroll
@@ -395,20 +421,21 @@ gca_bwd_gathered_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uin
 #pragma unroll
                 for (int db = 0; db < DB; ++db) {
                     const int o0 = tr.off(t4, db, RB);
-                    const bf16x8 b = lds_read_tr_pair(kb + o0, kb + o0 + 8 * RB);
+                    const bf16x8 b = lds_read_tr_pair(kbuf + o0, kbuf + o0 + 8 * RB);
                     dqacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, dsA[t4], dqacc[db], 0, 0, 0);
                 }
             __syncthreads();
-            // key block `wave`: lane = key 32*wave + n, slots = the 16 queries of step t4
+            // key block kb: lane = key 32*kb + n, slots = the 16 queries of step t (all G heads' rows in turn)
 #pragma unroll
-            for (int t4 = 0; t4 < 4; ++t4) {
-                const int o0 = tr.off(t4, wave, RB);
-                const bf16x8 pT = lds_read_tr_pair(xP + o0, xP + o0 + 8 * RB);
-                const bf16x8 sT = lds_read_tr_pair(xS + o0, xS + o0 + 8 * RB);
+            for (int ti = 0; ti < NTEN; ++ti) {
+                const unsigned char* src = (ten0 + ti) == 0 ? xS : xP;       // dk takes dS, dv takes P~
 #pragma unroll
-                for (int db = 0; db < DB; ++db) {
-                    dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(doT[t4][db], pT, dvacc[db], 0, 0, 0);
-                    dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qT[t4][db], sT, dkacc[db], 0, 0, 0);
+                for (int t = 0; t < T; ++t) {
+                    const int o0 = tr.off(t, kb, RB);
+                    const bf16x8 bT = lds_read_tr_pair(src + o0, src + o0 + 8 * RB);
+#pragma unroll
+                    for (int di = 0; di < NDB; ++di)
+                        acc[ti][di] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aT[ti][t][di], bT, acc[ti][di], 0, 0, 0);
                 }
             }
         }
@@ -416,38 +443,46 @@ gca_bwd_gathered_mfma_kernel(Params p, const uint16_t* __restrict__ q, const uin
         wait_async_tiles();
         __syncthreads();
 
-        // dk / dv of slot j.  The accumulators hold the lane's key row, registers 4a .. 4a+3 of block db being dims
+        // dk / dv of slot j.  The accumulators hold the lane's key row, registers 4a .. 4a+3 of a block being dims
         // 32*db + 8a + 4h + 0..3; stored like that, an instruction would touch 32 rows with 16 bytes each.  The
-        // wavefront's 32 rows go through its own rows of the exchange tiles instead (free until the next chunk's
-        // exchange, and no other wavefront touches them before the next barrier) and leave as 16-byte pieces, eight
-        // lanes to a 128-byte row: 1 KB contiguous per instruction.  Issued after the wait above, so the stores are
-        // long done when the next chunk's wait comes.
+        // rows go through the first 64 rows of the exchange tiles instead (free until the next chunk's exchange;
+        // a wavefront reads back only what it wrote itself, so no barrier) and leave as 16-byte pieces, eight
+        // lanes to a 128-byte row.  Issued after the wait above, so the stores are long done when the next
+        // chunk's wait comes.
         {
             const float vscale = live ? (mult < 0.f ? -1.f : 1.f) / p.sm_scale : 0.f;
-#pragma unroll
-            for (int db = 0; db < DB; ++db)
-#pragma unroll
-                for (int a = 0; a < 4; ++a) {
-                    union { __bf16 b[4]; uint64_t u; } pk, pv;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        pk.b[e] = (__bf16)dkacc[db][4 * a + e];
-                        pv.b[e] = (__bf16)(dvacc[db][4 * a + e] * vscale);
-                    }
-                    const int off = xrow + (((4 * db + a) ^ fsw) << 4);
-                    *reinterpret_cast<uint64_t*>(xP + off) = pk.u;
-                    *reinterpret_cast<uint64_t*>(xS + off) = pv.u;
-                }
             int64_t rs;
             const int64_t slot = chunk_base_n(p, k, nullptr, 0, z, hk, j, rs) - k;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int row = 32 * wave + 8 * i + (lane >> 3), lp = lane & 7;
-                const int off = tile_off(row, lp, RB);
-                const u32x4 kq = *reinterpret_cast<const u32x4*>(xP + off);
-                const u32x4 vq = *reinterpret_cast<const u32x4*>(xS + off);
-                *reinterpret_cast<u32x4*>(dk + slot + row * D + lp * 8) = kq;
-                *reinterpret_cast<u32x4*>(dv + slot + row * D + lp * 8) = vq;
+            for (int ti = 0; ti < NTEN; ++ti) {
+                const bool is_dv = (ten0 + ti) != 0;
+                unsigned char* stage = is_dv ? xS : xP;
+                uint16_t* out = (is_dv ? dv : dk) + slot;
+                const float sc = is_dv ? vscale : 1.f;
+#pragma unroll
+                for (int di = 0; di < NDB; ++di)
+#pragma unroll
+                    for (int a = 0; a < 4; ++a) {
+                        union { __bf16 b[4]; uint64_t u; } pk;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) pk.b[e] = (__bf16)(acc[ti][di][4 * a + e] * sc);
+                        *reinterpret_cast<uint64_t*>(stage + krow + (((4 * (db0 + di) + a) ^ fsw) << 4)) = pk.u;
+                    }
+                if constexpr (NDB == 2) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int row = 32 * kb + 8 * i + (lane >> 3), lp = lane & 7;
+                        const u32x4 val = *reinterpret_cast<const u32x4*>(stage + tile_off(row, lp, RB));
+                        *reinterpret_cast<u32x4*>(out + row * D + lp * 8) = val;
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 2; ++i) {
+                        const int row = 32 * kb + 16 * i + (lane >> 2), lp = 4 * db0 + (lane & 3);
+                        const u32x4 val = *reinterpret_cast<const u32x4*>(stage + tile_off(row, lp, RB));
+                        *reinterpret_cast<u32x4*>(out + row * D + lp * 8) = val;
+                    }
+                }
             }
         }
     }
@@ -1053,14 +1088,20 @@ static int launch_bwd_d(const Params& p, const void* q, const void* k, const voi
                         float* delta, void* lists, hipStream_t s) {
     int rc = GCA_OK;
     if constexpr (D == 64) {
-        // gathered form, one query head per kv head, one query tile: dq, dk and dv in one launch
+        // gathered form, one query tile, 1 / 2 / 4 query heads per kv head: dq, dk and dv in one launch
         const int both = GCA_STAGE_DQ | GCA_STAGE_DKDV;
-        if (!p.indexed && p.G == 1 && p.Q_CTX == 64 && (p.stages & both) == both) {
+        if (!p.indexed && (p.G == 1 || p.G == 2 || p.G == 4) && p.Q_CTX == 64 && (p.stages & both) == both) {
             const int64_t blocks = xcd_grid(p.Z * p.Hkv);
             if (blocks <= 0 || blocks > 0x7fffffffLL) return GCA_ERR_SHAPE;
-            hipLaunchKernelGGL((gca_bwd_gathered_mfma_kernel<D>), dim3((unsigned)blocks), dim3(128), 0, s, p,
-                               (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse,
-                               (uint16_t*)dq, (uint16_t*)dk, (uint16_t*)dv, delta);
+            const dim3 grid((unsigned)blocks);
+#define GCA_LAUNCH_GATHERED(GG)                                                                                         \
+            hipLaunchKernelGGL((gca_bwd_gathered_mfma_kernel<D, GG>), grid, dim3(128 * GG), 0, s, p, (const uint16_t*)q, \
+                               (const uint16_t*)k, (const uint16_t*)v, w, wb, (const uint16_t*)dout, lse, (uint16_t*)dq, \
+                               (uint16_t*)dk, (uint16_t*)dv, delta)
+            if (p.G == 1) GCA_LAUNCH_GATHERED(1);
+            else if (p.G == 2) GCA_LAUNCH_GATHERED(2);
+            else GCA_LAUNCH_GATHERED(4);
+#undef GCA_LAUNCH_GATHERED
             if (hipGetLastError() != hipSuccess) return GCA_ERR_LAUNCH;
             return (p.stages & GCA_STAGE_DW) ? launch_dw(p, delta, dw, s) : GCA_OK;
         }

@@ -1,5 +1,5 @@
-"""Gathered-form backward in one launch (bf16, d = 64, one query head per kv head, 64 query rows): dq, dk and dv
-from the same pass over K / V.
+"""Gathered-form backward in one launch (bf16, d = 64, 1 / 2 / 4 query heads per kv head, 64 query rows): dq, dk and
+dv from the same pass over K / V.
 
 Checked against the oracle like every other path, and against the staged form of the same entry point
 (``desc.stages`` = dq alone, then dk/dv alone, which runs the two separate kernels): both round P and dS to bf16 once
@@ -38,11 +38,13 @@ def _bwd(q, k, v, w, do, lse, sm_scale, stages_seq):
 
 
 @pytest.mark.parametrize("w_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("Z,H,K", [(3, 2, 1), (5, 3, 3), (7, 12, 8), (2, 1, 16), (64, 4, 5)])
-def test_one_launch_equals_staged_form_and_oracle(Z, H, K, w_dtype):
+@pytest.mark.parametrize("Z,Hq,Hkv,K", [(3, 2, 2, 1), (5, 3, 3, 3), (7, 12, 12, 8), (2, 1, 1, 16), (64, 4, 4, 5),
+                                        (5, 4, 2, 3), (4, 2, 1, 5), (9, 6, 3, 8),          # two query heads per kv head
+                                        (3, 8, 2, 4), (6, 4, 1, 8), (17, 12, 3, 2)])       # four
+def test_one_launch_equals_staged_form_and_oracle(Z, Hq, Hkv, K, w_dtype):
     from gca_hip.gca import _forward
     S, d = 64, 64
-    q, k, v, w, do = gca_inputs(Z, H, H, K, S, S, d, torch.bfloat16, seed=900 + Z + K, w_dtype=torch.float32)
+    q, k, v, w, do = gca_inputs(Z, Hq, Hkv, K, S, S, d, torch.bfloat16, seed=900 + Z + K, w_dtype=torch.float32)
     g = torch.Generator().manual_seed(901 + K)
     w = torch.randn(Z, K, generator=g)
     if K > 1:
