@@ -182,8 +182,10 @@ def kernel_times(torch, q, ck, cv, idx, w, do, sm_scale, sm_n, iters):
 def run_cfg2_gathered(torch, dev, seed, iters):
     """Config 2 through the drop-in call the reference's model makes (model/DRT.py:380): attention(q, k, v, weights,
     ...) on gathered, K-times-larger copies of the retrieved chunks, forward + backward.  Here the K-fold bytes are
-    real HBM traffic.  `with_gather` adds the reference-style gather copies (model/DRT.py:193-200, :320-332) and
-    autograd's scatter-add of dk/dv back into the cache."""
+    real HBM traffic.  `with_reference_style_gather_and_scatter` adds what produces and consumes those copies around
+    the call: the gather of the retrieved chunks into the reference's layout (model/DRT.py:193-200, :320-332; here
+    one kernel, `gca_gather_chunks`) and, in the backward, the sum of dk/dv back into the cache (autograd's
+    index_put_(accumulate=True) in the reference; here `gca_scatter_chunks`)."""
     import gca_hip
     N, C, H, S, d, K = 8, 256, 12, 64, 64, 8
     q, ck, cv, lq, lk, do = cfg2_inputs(torch, dev, seed)

@@ -136,6 +136,37 @@ typedef struct chunk_cache_desc {
     int32_t reserved;
 } chunk_cache_desc;
 
+/* Shape of a gather of retrieved chunks: cache (N, C, S, Hkv*D), indices (Z, K) with row z belonging to sequence
+ * z / (Z/N), gathered tensors (Z, Hkv, K, S, D).  D * element size must be a multiple of 16 bytes. */
+typedef struct chunk_gather_desc {
+    int32_t dtype;          /* gca_dtype of the caches and the gathered tensors */
+    int32_t Hkv;            /* heads the cache rows are split into (1: rows stay whole, D = the full width) */
+    int64_t N;              /* sequences */
+    int64_t C;              /* chunks per sequence in the cache */
+    int64_t Z;              /* index rows, a multiple of N */
+    int32_t K;              /* indices per row */
+    int32_t S;              /* rows per chunk */
+    int32_t D;              /* width of a head row */
+    int32_t reserved;
+} chunk_gather_desc;
+
+/* k_out[z, h, j, s, :] = k_cache[n, indices[z, j], s, h*D : (h+1)*D] (same for v) in one pass over the data:
+ * ChunkKVManager.retrieve_chunks (model/DRT.py:193-200, advanced indexing) followed by the rearrange
+ * 'N (D K) S (h d) -> (N D) h K S d' + contiguous of preprocess_chunk_kv_cache (model/DRT.py:320-332), which the
+ * reference runs as two K-times-larger copies per tensor.  With Hkv = 1 and D = the full row width it is
+ * retrieve_chunks alone.  Ids outside [0, C) are clamped.  Only callers of the gathered kernels need it. */
+int gca_gather_chunks(const chunk_gather_desc* desc, const void* k_cache, const void* v_cache, const int64_t* indices,
+                      void* k_out, void* v_out, void* stream);
+
+/* Backward of gca_gather_chunks: dk_cache[n, c] = sum of dk[z, :, j] over the (z, j) that retrieved chunk c (same
+ * for dv), what autograd's index_put_(accumulate=True) computes for the reference's advanced indexing
+ * (model/DRT.py:198-199), but walked in a fixed order with float accumulation: every cache element is written
+ * exactly once (zeros where nobody retrieved the chunk), no atomics, no zero-fill, same bits every run.
+ * workspace: gca_scatter_workspace_bytes(desc) bytes (the reference lists are built there). */
+size_t gca_scatter_workspace_bytes(const chunk_gather_desc* desc);
+int gca_scatter_chunks(const chunk_gather_desc* desc, const void* dk, const void* dv, const int64_t* indices,
+                       void* dk_cache, void* dv_cache, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Library version (major*10000 + minor*100 + patch; 200: lmk_desc has chunk_win) and status text. */
 int gca_version(void);
 const char* gca_strerror(int status);

@@ -1,9 +1,10 @@
-// Append kernel of the device-resident chunk cache: new chunks are copied into their slots of a cache
+// Kernels of the device-resident chunk cache.  Append: new chunks are copied into their slots of a cache
 // allocated with spare capacity, with the landmark row of every chunk kept, zeroed or dropped on the way.
 // Pure data movement, bound by HBM: every workgroup moves 16-byte vectors, consecutive lanes touching
 // consecutive addresses on both sides.
 #include "gca_common.h"
 #include "gca_mfma.h"
+#include "gca_lists.h"
 
 namespace gca {
 
@@ -86,6 +87,175 @@ int launch_chunk_append(const chunk_cache_desc& d, const void* sk, const void* s
     if (d.dtype == GCA_F32) return launch_append_t<float>(d, a, sk, sv, sl, dk, dv, dl, s);
     if (d.dtype == GCA_BF16) return launch_append_t<uint16_t>(d, a, sk, sv, sl, dk, dv, dl, s);
     return GCA_ERR_DTYPE;
+}
+
+// ------------------------------------------------------------------- gather / scatter of retrieved chunks
+//
+// Gather: out[z, hk, j, s, :] = cache[n(z), indices[z, j], s, hk*D : (hk+1)*D] for K and V in one pass -- the
+// advanced-index copy and the rearrange + contiguous copy of the reference done as one.  One workgroup column per
+// (z, j); a chunk is S rows of Hkv * ppr 16-byte pieces, read in row order (consecutive lanes, consecutive
+// addresses) and written head by head (ppr lanes to a contiguous head row).
+// Scatter (its backward): dcache[n, c, s, hk*D:] = sum over the references (z, j) with indices[z, j] == c of
+// d[z, hk, j, s, :], walked in the reference lists' fixed order, accumulated in float, every cache element
+// written exactly once (zeros where nobody retrieved the chunk): no atomics, no zero-fill, same bits every run.
+
+namespace {
+
+struct GatherArgs {
+    int64_t N, C, Z, zpn;
+    int K, S, Hkv, D;
+    int ppr;          // 16-byte pieces per head row
+};
+
+__global__ void __launch_bounds__(256)
+chunk_gather_kernel(GatherArgs a, const u32x4* __restrict__ k_cache, const u32x4* __restrict__ v_cache,
+                    const int64_t* __restrict__ indices, u32x4* __restrict__ k_out, u32x4* __restrict__ v_out) {
+    const int64_t zj = blockIdx.x;
+    const int64_t z = zj / a.K;
+    const int j = (int)(zj % a.K);
+    const int64_t n = z / a.zpn;
+    const int64_t c = clamp_idx(indices[zj], a.C);
+    const int row = a.Hkv * a.ppr;                       // pieces per cache row
+    const int64_t src0 = (n * a.C + c) * a.S * row;
+    const int total = a.S * row;
+    for (int i = blockIdx.y * 256 + threadIdx.x; i < total; i += gridDim.y * 256) {
+        const int s = i / row, r = i - s * row;
+        const int hk = r / a.ppr, pp = r - hk * a.ppr;
+        const int64_t dst = (((z * a.Hkv + hk) * a.K + j) * a.S + s) * a.ppr + pp;
+        k_out[dst] = k_cache[src0 + i];
+        v_out[dst] = v_cache[src0 + i];
+    }
+}
+
+template <typename E> __device__ __forceinline__ float piece_elem(const u32x4& v, int e);
+template <> __device__ __forceinline__ float piece_elem<float>(const u32x4& v, int e) { return __uint_as_float(v[e]); }
+template <> __device__ __forceinline__ float piece_elem<uint16_t>(const u32x4& v, int e) {
+    const uint32_t word = v[e >> 1];
+    return __uint_as_float((e & 1) ? (word & 0xffff0000u) : (word << 16));
+}
+
+constexpr int SCATTER_BATCH = 256;      // references whose tile offsets are staged in LDS at a time
+
+template <typename E>
+__global__ void __launch_bounds__(256)
+chunk_scatter_kernel(GatherArgs a, const E* __restrict__ dk_g, const E* __restrict__ dv_g, E* __restrict__ dk_cache,
+                     E* __restrict__ dv_cache, ListWs ws) {
+    constexpr int V = 16 / sizeof(E);
+    __shared__ int64_t s_tile[SCATTER_BATCH];            // element offset of the reference's (z, hk, j) tile
+    const int tid = threadIdx.x;
+    const int64_t cc = blockIdx.x / a.Hkv;
+    const int hk = (int)(blockIdx.x % a.Hkv);
+    const int nref = ws.count[cc], list0 = ws.start[cc];
+    const int tile = a.S * a.D;
+    const int pieces = tile / V;
+    // a thread owns pieces tid, tid + 256, ...; NP of them are carried through a batch of references at a time
+    constexpr int NP = 4;
+    for (int pbase = 0; pbase < pieces; pbase += 256 * NP) {      // uniform bounds: the loop body has barriers
+        const int p0 = pbase + tid;
+        float acc_k[NP][V], acc_v[NP][V];
+#pragma unroll
+        for (int q = 0; q < NP; ++q)
+#pragma unroll
+            for (int e = 0; e < V; ++e) { acc_k[q][e] = 0.f; acc_v[q][e] = 0.f; }
+        for (int r0 = 0; r0 < nref; r0 += SCATTER_BATCH) {
+            const int nb = min(SCATTER_BATCH, nref - r0);
+            __syncthreads();
+            if (tid < nb) {
+                const int64_t z = ws.ref_zj[2 * (list0 + r0 + tid)], j = ws.ref_zj[2 * (list0 + r0 + tid) + 1];
+                s_tile[tid] = ((z * a.Hkv + hk) * a.K + j) * (int64_t)tile;
+            }
+            __syncthreads();
+            for (int ri = 0; ri < nb; ++ri) {
+                const int64_t base = s_tile[ri];
+#pragma unroll
+                for (int q = 0; q < NP; ++q) {
+                    const int piece = p0 + 256 * q;
+                    if (piece < pieces) {
+                        const u32x4 kv = *reinterpret_cast<const u32x4*>(dk_g + base + (int64_t)piece * V);
+                        const u32x4 vv = *reinterpret_cast<const u32x4*>(dv_g + base + (int64_t)piece * V);
+#pragma unroll
+                        for (int e = 0; e < V; ++e) {
+                            acc_k[q][e] += piece_elem<E>(kv, e);
+                            acc_v[q][e] += piece_elem<E>(vv, e);
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < NP; ++q) {
+            const int piece = p0 + 256 * q;
+            if (piece < pieces) {
+                const int el = piece * V, s = el / a.D, col = el - s * a.D;
+                const int64_t dst = ((cc * a.S + s) * a.Hkv + hk) * (int64_t)a.D + col;
+                union { E e[V]; u32x4 v; } ok, ov;
+#pragma unroll
+                for (int e = 0; e < V; ++e) {
+                    if constexpr (sizeof(E) == 2) {
+                        ok.e[e] = f_to_bf16_bits(acc_k[q][e]);
+                        ov.e[e] = f_to_bf16_bits(acc_v[q][e]);
+                    } else {
+                        ok.e[e] = acc_k[q][e];
+                        ov.e[e] = acc_v[q][e];
+                    }
+                }
+                *reinterpret_cast<u32x4*>(dk_cache + dst) = ok.v;
+                *reinterpret_cast<u32x4*>(dv_cache + dst) = ov.v;
+            }
+        }
+    }
+}
+
+GatherArgs gather_args(const chunk_gather_desc& d) {
+    GatherArgs a;
+    a.N = d.N; a.C = d.C; a.Z = d.Z; a.zpn = d.Z / d.N;
+    a.K = d.K; a.S = d.S; a.Hkv = d.Hkv; a.D = d.D;
+    a.ppr = d.D * (d.dtype == GCA_F32 ? 4 : 2) / 16;
+    return a;
+}
+
+// the list builders only look at the retrieval's shape
+Params list_params(const chunk_gather_desc& d) {
+    Params p = {};
+    p.Z = d.Z; p.N = d.N; p.C = d.C; p.zpn = d.Z / d.N; p.K = d.K;
+    p.Hkv = d.Hkv; p.K_CTX = d.S; p.D = d.D; p.indexed = 1;
+    return p;
+}
+
+constexpr int SCATTER_SEG_MAX = 1 << 30;     // the scatter walks every chunk's list whole
+
+}  // namespace
+
+int launch_chunk_gather(const chunk_gather_desc& d, const void* k_cache, const void* v_cache, const int64_t* indices,
+                        void* k_out, void* v_out, hipStream_t s) {
+    const GatherArgs a = gather_args(d);
+    const int64_t cols = d.Z * d.K;
+    if (cols > INT32_MAX || (int64_t)a.S * a.Hkv * a.ppr > INT32_MAX) return GCA_ERR_SHAPE;
+    int64_t by = ((int64_t)a.S * a.Hkv * a.ppr + 256 * 8 - 1) / (256 * 8);      // about 8 pieces per thread
+    by = by < 1 ? 1 : (by > 64 ? 64 : by);
+    hipLaunchKernelGGL(chunk_gather_kernel, dim3((unsigned)cols, (unsigned)by), dim3(256), 0, s, a, (const u32x4*)k_cache,
+                       (const u32x4*)v_cache, indices, (u32x4*)k_out, (u32x4*)v_out);
+    return hipGetLastError() == hipSuccess ? GCA_OK : GCA_ERR_LAUNCH;
+}
+
+size_t chunk_scatter_ws_bytes(const chunk_gather_desc& d) { return list_table_bytes(list_params(d), SCATTER_SEG_MAX); }
+
+int launch_chunk_scatter(const chunk_gather_desc& d, const void* dk_g, const void* dv_g, const int64_t* indices,
+                         void* dk_cache, void* dv_cache, void* workspace, hipStream_t s) {
+    const Params p = list_params(d);
+    const ListWs ws = list_carve(p, SCATTER_SEG_MAX, workspace, nullptr);
+    int rc = list_build(p, SCATTER_SEG_MAX, indices, ws, s);
+    if (rc != GCA_OK) return rc;
+    const GatherArgs a = gather_args(d);
+    const int64_t blocks = d.N * d.C * d.Hkv;
+    if (blocks > INT32_MAX) return GCA_ERR_SHAPE;
+    if (d.dtype == GCA_F32)
+        hipLaunchKernelGGL((chunk_scatter_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, s, a, (const float*)dk_g,
+                           (const float*)dv_g, (float*)dk_cache, (float*)dv_cache, ws);
+    else
+        hipLaunchKernelGGL((chunk_scatter_kernel<uint16_t>), dim3((unsigned)blocks), dim3(256), 0, s, a, (const uint16_t*)dk_g,
+                           (const uint16_t*)dv_g, (uint16_t*)dk_cache, (uint16_t*)dv_cache, ws);
+    return hipGetLastError() == hipSuccess ? GCA_OK : GCA_ERR_LAUNCH;
 }
 
 }  // namespace gca

@@ -278,4 +278,41 @@ int chunk_cache_append(const chunk_cache_desc* d, const void* src_k, const void*
     return launch_chunk_append(*d, src_k, src_v, src_lmk, k_cache, v_cache, lmk_cache, (hipStream_t)stream);
 }
 
+static int check_gather(const chunk_gather_desc* d) {
+    if (d == nullptr) return GCA_ERR_NULL;
+    if (d->dtype != GCA_F32 && d->dtype != GCA_BF16) return GCA_ERR_DTYPE;
+    if (d->N <= 0 || d->C <= 0 || d->Z <= 0 || d->K <= 0 || d->S <= 0 || d->D <= 0 || d->Hkv <= 0) return GCA_ERR_SHAPE;
+    if (d->Z % d->N != 0) return GCA_ERR_SHAPE;
+    if (((int64_t)d->D * (d->dtype == GCA_F32 ? 4 : 2)) % 16 != 0) return GCA_ERR_SHAPE;
+    return GCA_OK;
+}
+
+static bool aligned16(const void* a, const void* b, const void* c, const void* d) {
+    return (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)d) % 16) == 0;
+}
+
+int gca_gather_chunks(const chunk_gather_desc* desc, const void* k_cache, const void* v_cache, const int64_t* indices,
+                      void* k_out, void* v_out, void* stream) {
+    int rc = check_gather(desc);
+    if (rc != GCA_OK) return rc;
+    if (!k_cache || !v_cache || !indices || !k_out || !v_out) return GCA_ERR_NULL;
+    if (!aligned16(k_cache, v_cache, k_out, v_out)) return GCA_ERR_SHAPE;
+    return launch_chunk_gather(*desc, k_cache, v_cache, indices, k_out, v_out, (hipStream_t)stream);
+}
+
+size_t gca_scatter_workspace_bytes(const chunk_gather_desc* desc) {
+    if (check_gather(desc) != GCA_OK) return 0;
+    return chunk_scatter_ws_bytes(*desc);
+}
+
+int gca_scatter_chunks(const chunk_gather_desc* desc, const void* dk, const void* dv, const int64_t* indices,
+                       void* dk_cache, void* dv_cache, void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_gather(desc);
+    if (rc != GCA_OK) return rc;
+    if (!dk || !dv || !indices || !dk_cache || !dv_cache) return GCA_ERR_NULL;
+    if (!aligned16(dk, dv, dk_cache, dv_cache)) return GCA_ERR_SHAPE;
+    if (!workspace || workspace_bytes < chunk_scatter_ws_bytes(*desc)) return GCA_ERR_WORKSPACE;
+    return launch_chunk_scatter(*desc, dk, dv, indices, dk_cache, dv_cache, workspace, (hipStream_t)stream);
+}
+
 }  // extern "C"

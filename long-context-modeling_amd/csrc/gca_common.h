@@ -128,6 +128,11 @@ int launch_lmk_bwd(const lmk_desc& d, const void* lq, const void* lk, const int6
 size_t bwd_workspace_bytes(const gca_desc& d, bool indexed);
 int launch_chunk_append(const chunk_cache_desc& d, const void* sk, const void* sv, const void* sl,
                         void* dk, void* dv, void* dl, hipStream_t s);
+int launch_chunk_gather(const chunk_gather_desc& d, const void* k_cache, const void* v_cache, const int64_t* indices,
+                        void* k_out, void* v_out, hipStream_t s);
+size_t chunk_scatter_ws_bytes(const chunk_gather_desc& d);
+int launch_chunk_scatter(const chunk_gather_desc& d, const void* dk_g, const void* dv_g, const int64_t* indices,
+                         void* dk_cache, void* dv_cache, void* workspace, hipStream_t s);
 int launch_dw(const Params& p, const float* delta, float* dw, hipStream_t s);
 // bytes of the per-chunk row sums D_j at the start of the backward workspace (256-byte multiple)
 inline size_t delta_bytes(const Params& p) {

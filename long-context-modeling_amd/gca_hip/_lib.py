@@ -24,6 +24,7 @@ SYMBOLS = (
     "gca_bwd_indexed", "lmk_score", "lmk_topk_workspace_bytes", "lmk_topk", "lmk_score_topk",
     "lmk_weights_bwd_workspace_bytes", "lmk_weights_bwd", "chunk_cache_append", "lmk_score_topk_static",
     "gca_lists_workspace_bytes", "gca_lists_build", "gca_bwd_indexed_lists",
+    "gca_gather_chunks", "gca_scatter_workspace_bytes", "gca_scatter_chunks",
 )
 LMK_STATIC_SCRATCH_BYTES = 8 << 20
 GCA_ERR_UNSUPPORTED = 6
@@ -52,6 +53,14 @@ class LmkDesc(ctypes.Structure):
         ("N", ctypes.c_int64), ("C", ctypes.c_int64), ("E", ctypes.c_int64),
         ("Dm", ctypes.c_int32), ("causal", ctypes.c_int32),
         ("hidden_size", ctypes.c_float), ("lmk_k_rows", ctypes.c_int32), ("chunk_win", ctypes.c_int32),
+    ]
+
+
+class ChunkGatherDesc(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int32), ("Hkv", ctypes.c_int32),
+        ("N", ctypes.c_int64), ("C", ctypes.c_int64), ("Z", ctypes.c_int64),
+        ("K", ctypes.c_int32), ("S", ctypes.c_int32), ("D", ctypes.c_int32), ("reserved", ctypes.c_int32),
     ]
 
 
@@ -104,6 +113,13 @@ def _declare(lib):
     lib.lmk_weights_bwd_workspace_bytes.argtypes = [L]
     lib.lmk_weights_bwd.restype = ctypes.c_int
     lib.lmk_weights_bwd.argtypes = [L, P, P, I64P, FP, FP, P, P, P, ctypes.c_size_t, P]
+    G = ctypes.POINTER(ChunkGatherDesc)
+    lib.gca_gather_chunks.restype = ctypes.c_int
+    lib.gca_gather_chunks.argtypes = [G, P, P, I64P, P, P, P]
+    lib.gca_scatter_workspace_bytes.restype = ctypes.c_size_t
+    lib.gca_scatter_workspace_bytes.argtypes = [G]
+    lib.gca_scatter_chunks.restype = ctypes.c_int
+    lib.gca_scatter_chunks.argtypes = [G, P, P, I64P, P, P, P, ctypes.c_size_t, P]
     lib.chunk_cache_append.restype = ctypes.c_int
     lib.chunk_cache_append.argtypes = [ctypes.POINTER(ChunkCacheDesc), P, P, P, P, P, P, P]
 

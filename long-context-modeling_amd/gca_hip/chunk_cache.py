@@ -17,7 +17,7 @@ import torch
 
 from . import _lib
 from .gca import _DT, _ptr, _stream, gca_kv_cache, gca_kv_cache_indexed
-from .retrieval import landmark_retrieve
+from .retrieval import gather_rows, landmark_retrieve
 
 _LMK_ROW = {"keep": _lib.CHUNK_LMK_KEEP, "zero": _lib.CHUNK_LMK_ZERO, "drop": _lib.CHUNK_LMK_DROP}
 
@@ -216,8 +216,7 @@ class ChunkKVManager:
         """k, v = cache[n, indices[n, i]] -> (N, len, S, Dm) (DRT.py:193-220)."""
         N = indices.shape[0]
         if not self._offloading:
-            b = torch.arange(N, device=indices.device).unsqueeze(1)
-            return self.chunk_k[b, indices], self.chunk_v[b, indices]
+            return gather_rows(self.chunk_k, self.chunk_v, indices)
         ci = indices.cpu()
         b = torch.arange(N).unsqueeze(1)
         # gather into pinned staging so the copy to the device is one asynchronous transfer per tensor

@@ -215,22 +215,88 @@ def landmark_retrieve_static(lmk_q, lmk_k, topk, out_indices, out_weights, hidde
     return out_indices, out_weights
 
 
+def _gather_desc(cache, Z, K, num_kv_heads, chunks_allocated=None):
+    N, C, S, Dm = cache.shape
+    assert Dm % num_kv_heads == 0 and Z % N == 0
+    return _lib.ChunkGatherDesc(dtype=_DT[cache.dtype], Hkv=num_kv_heads, N=N, C=chunks_allocated or C, Z=Z, K=K, S=S,
+                                D=Dm // num_kv_heads)
+
+
+def _chunks_allocated(t):
+    """Chunks per sequence in the memory behind ``t`` (N, C, S, Dm): C for a dense tensor, the capacity for the
+    filled part ``store[:, :C]`` of a store with spare room (read in place), None for any other layout."""
+    N, C, S, Dm = t.shape
+    if t.is_contiguous():
+        return C
+    s0, s1, s2, s3 = t.stride()
+    if s3 == 1 and s2 == Dm and s1 == S * Dm and s0 % (S * Dm) == 0 and s0 // (S * Dm) >= C:
+        return s0 // (S * Dm)
+    return None
+
+
+class _GatherChunks(torch.autograd.Function):
+    """cache (N, C, S, Hkv*d) x idx (Z, K) -> (Z, Hkv, K, S, d) for K and V in one kernel; the backward sums the
+    gathered gradients back into cache-shaped tensors in a fixed order (``gca_scatter_chunks``)."""
+
+    @staticmethod
+    def forward(ctx, chunk_k, chunk_v, idx, num_kv_heads):
+        assert chunk_k.is_cuda and chunk_k.dim() == 4 and chunk_k.shape == chunk_v.shape and chunk_k.dtype in _DT
+        assert chunk_v.dtype == chunk_k.dtype and idx.dtype == torch.int64 and idx.dim() == 2
+        idx = idx.contiguous()
+        alloc = _chunks_allocated(chunk_k)
+        if alloc is None or alloc != _chunks_allocated(chunk_v):
+            chunk_k, chunk_v, alloc = chunk_k.contiguous(), chunk_v.contiguous(), chunk_k.shape[1]
+        N, C, S, Dm = chunk_k.shape
+        Z, K = idx.shape
+        desc = _gather_desc(chunk_k, Z, K, num_kv_heads, alloc)
+        shape = (Z, num_kv_heads, K, S, Dm // num_kv_heads)
+        k_out = torch.empty(shape, device=chunk_k.device, dtype=chunk_k.dtype)
+        v_out = torch.empty(shape, device=chunk_k.device, dtype=chunk_k.dtype)
+        with torch.cuda.device(chunk_k.device):
+            rc = _lib.lib().gca_gather_chunks(ctypes.byref(desc), _ptr(chunk_k), _ptr(chunk_v), _ptr(idx), _ptr(k_out),
+                                              _ptr(v_out), _stream(chunk_k.device))
+        _lib.check(rc, "gca_gather_chunks")
+        ctx.save_for_backward(idx)
+        ctx.cache_shape, ctx.heads = tuple(chunk_k.shape), num_kv_heads
+        return k_out, v_out
+
+    @staticmethod
+    def backward(ctx, dk, dv):
+        idx, = ctx.saved_tensors
+        dk, dv = dk.contiguous(), dv.contiguous()
+        dkc = torch.empty(ctx.cache_shape, device=dk.device, dtype=dk.dtype)
+        dvc = torch.empty(ctx.cache_shape, device=dk.device, dtype=dk.dtype)
+        desc = _gather_desc(dkc, idx.shape[0], idx.shape[1], ctx.heads)
+        with torch.cuda.device(dk.device):
+            L = _lib.lib()
+            nbytes = L.gca_scatter_workspace_bytes(ctypes.byref(desc))
+            ws = torch.empty(nbytes // 4 + 1, device=dk.device, dtype=torch.int32)
+            rc = L.gca_scatter_chunks(ctypes.byref(desc), _ptr(dk), _ptr(dv), _ptr(idx), _ptr(dkc), _ptr(dvc), _ptr(ws),
+                                      nbytes, _stream(dk.device))
+        _lib.check(rc, "gca_scatter_chunks")
+        return dkc, dvc, None, None
+
+
+def gather_rows(chunk_k, chunk_v, indices):
+    """k, v = cache[n, indices[n, i]] -> (N, len, S, Dm): ``ChunkKVManager.retrieve_chunks`` (model/DRT.py:193-200)
+    as one kernel for both tensors, with the deterministic scatter as its backward."""
+    N, L = indices.shape
+    S, Dm = chunk_k.shape[2], chunk_k.shape[3]
+    k, v = _GatherChunks.apply(chunk_k, chunk_v, indices, 1)          # (N, 1, L, S, Dm)
+    return k.view(N, L, S, Dm), v.view(N, L, S, Dm)
+
+
 def gather_chunks(chunk_k, chunk_v, indices, weights, num_kv_heads):
-    """The reference's gather + layout (model/DRT.py:198-199, :629-637, :328-332): drops the
-    last retrieval row and returns k, v ((N (C-1)), Hkv, K, S, d) and weights ((N (C-1)), K).
-    Only needed by callers of the gathered-form ``attention``; ``attention_indexed`` reads the
-    cache directly."""
+    """The reference's gather + layout (model/DRT.py:198-199, :629-637, :328-332) in one kernel: drops the
+    last retrieval row and returns k, v ((N (C-1)), Hkv, K, S, d) and weights ((N (C-1)), K).  Gradients of k and v
+    flow back into the caches through a deterministic scatter (the reference gets there through autograd's
+    ``index_put_(accumulate=True)``).  Only needed by callers of the gathered-form ``attention``;
+    ``attention_indexed`` reads the cache directly."""
     N, C, S, Dm = chunk_k.shape
     K = indices.shape[-1]
-    d = Dm // num_kv_heads
-    idx = indices[:, :-1, :].reshape(N, (C - 1) * K)
-    bidx = torch.arange(N, device=chunk_k.device).unsqueeze(1)
-
-    def g(cache):
-        x = cache[bidx, idx].view(N, C - 1, K, S, num_kv_heads, d)
-        return x.permute(0, 1, 4, 2, 3, 5).reshape(N * (C - 1), num_kv_heads, K, S, d).contiguous()
-
-    return g(chunk_k), g(chunk_v), weights[:, :-1, :].reshape(N * (C - 1), K).contiguous()
+    idx = indices[:, :-1, :].reshape(N * (C - 1), K)
+    k, v = _GatherChunks.apply(chunk_k, chunk_v, idx, num_kv_heads)
+    return k, v, weights[:, :-1, :].reshape(N * (C - 1), K).contiguous()
 
 
 def gca_layer(q_all, chunk_k, chunk_v, lmk_q, lmk_k, topk, sm_n=0.0, hidden_size=None, noise=None, training=True):

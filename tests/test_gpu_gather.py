@@ -1,0 +1,133 @@
+"""The reference's gather of retrieved chunks (``ChunkKVManager.retrieve_chunks`` model/DRT.py:193-200 + the layout
+change of ``preprocess_chunk_kv_cache`` :320-332) as one kernel, and its backward as a deterministic scatter.
+
+The gather moves bits, so it is compared bit for bit with the oracle's advanced indexing + rearrange.  The scatter
+is a sum: against autograd through the oracle's gather in float64, to fp32 / bf16 rounding; run twice it must give
+the same bits; chunks nobody retrieved get exact zeros; a chunk retrieved by every row (a list longer than one batch
+of staged references) and ids outside the cache (clamped, as in the indexed kernels) are covered.
+"""
+import ctypes
+
+import pytest
+import torch
+
+from helpers import gen
+from oracle import gca_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _case(N, C, S, Dm, K, dtype, seed):
+    ck = gen((N, C, S, Dm), seed, 0.5, dtype)
+    cv = gen((N, C, S, Dm), seed + 1, 0.5, dtype)
+    g = torch.Generator().manual_seed(seed + 2)
+    idx = torch.randint(0, C, (N, C, K), generator=g)
+    w = torch.rand(N, C, K, generator=g)
+    return ck, cv, idx, w
+
+
+SHAPES = [(2, 5, 64, 128, 2, 3), (1, 9, 64, 768, 12, 8), (3, 4, 16, 64, 1, 2), (2, 7, 64, 64, 4, 1), (1, 33, 8, 512, 2, 5)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("N,C,S,Dm,Hkv,K", SHAPES)
+def test_gather_is_the_oracles_gather_bit_for_bit(N, C, S, Dm, Hkv, K, dtype):
+    import gca_hip
+    ck, cv, idx, w = _case(N, C, S, Dm, K, dtype, 10 + C)
+    k_o, v_o, w_o = orc.gather_chunks(ck, cv, idx, w, Hkv)
+    k, v, wg = gca_hip.gather_chunks(ck.to(DEV), cv.to(DEV), idx.to(DEV), w.to(DEV), Hkv)
+    assert k.shape == k_o.shape and k.is_contiguous() and v.is_contiguous()
+    assert torch.equal(k.cpu(), k_o) and torch.equal(v.cpu(), v_o) and torch.equal(wg.cpu(), w_o)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.bfloat16, 4e-3)])
+@pytest.mark.parametrize("N,C,S,Dm,Hkv,K", SHAPES)
+def test_scatter_is_the_gathers_gradient(N, C, S, Dm, Hkv, K, dtype, tol):
+    import gca_hip
+    ck, cv, idx, w = _case(N, C, S, Dm, K, dtype, 30 + C)
+    Z, d = N * (C - 1), Dm // Hkv
+    gk = gen((Z, Hkv, K, S, d), 40, 1.0, dtype)
+    gv = gen((Z, Hkv, K, S, d), 41, 1.0, dtype)
+    # autograd through the oracle's gather, in float64 on the same (already rounded) values
+    ck_o, cv_o = ck.double().requires_grad_(), cv.double().requires_grad_()
+    k_o, v_o, _ = orc.gather_chunks(ck_o, cv_o, idx, w.double(), Hkv)
+    torch.autograd.backward((k_o, v_o), (gk.double(), gv.double()))
+    ck_g, cv_g = ck.to(DEV).requires_grad_(), cv.to(DEV).requires_grad_()
+    k, v, _ = gca_hip.gather_chunks(ck_g, cv_g, idx.to(DEV), w.to(DEV), Hkv)
+    torch.autograd.backward((k, v), (gk.to(DEV), gv.to(DEV)))
+    for got, ref in ((ck_g.grad, ck_o.grad), (cv_g.grad, cv_o.grad)):
+        assert got.dtype == dtype and got.shape == ref.shape
+        scale = max(1.0, ref.abs().max().item())
+        assert (got.double().cpu() - ref).abs().max().item() <= tol * scale
+    unused = torch.ones(N, C, dtype=torch.bool)
+    unused[torch.arange(N).view(N, 1, 1).expand(N, C - 1, K), idx[:, :-1]] = False
+    assert (ck_g.grad.cpu()[unused] == 0).all() and (cv_g.grad.cpu()[unused] == 0).all()
+    # same bits on a second run
+    ck_g.grad = None
+    k2, v2, _ = gca_hip.gather_chunks(ck_g, cv_g, idx.to(DEV), w.to(DEV), Hkv)
+    first = cv_g.grad.clone()
+    cv_g.grad = None
+    torch.autograd.backward((k2, v2), (gk.to(DEV), gv.to(DEV)))
+    assert torch.equal(cv_g.grad, first)
+
+
+def test_chunk_retrieved_by_every_row_and_ids_outside_the_cache():
+    import gca_hip
+    N, C, S, Dm, Hkv, K = 1, 400, 16, 64, 2, 2
+    ck, cv, idx, w = _case(N, C, S, Dm, K, torch.bfloat16, 77)
+    idx[:, :, 0] = 3                         # a list of 399 references: more than one staged batch
+    idx[0, 5, 1] = C + 9                     # clamped to the last chunk
+    idx[0, 6, 1] = -4                        # clamped to chunk 0
+    clamped = idx.clamp(0, C - 1)
+    k_o, v_o, _ = orc.gather_chunks(ck, cv, clamped, w, Hkv)
+    ck_g, cv_g = ck.to(DEV).requires_grad_(), cv.to(DEV).requires_grad_()
+    k, v, _ = gca_hip.gather_chunks(ck_g, cv_g, idx.to(DEV), w.to(DEV), Hkv)
+    assert torch.equal(k.cpu(), k_o) and torch.equal(v.cpu(), v_o)
+    gk = gen(tuple(k.shape), 78, 1.0, torch.bfloat16)
+    ck_o = ck.double().requires_grad_()
+    k_o2, _, _ = orc.gather_chunks(ck_o, cv.double(), clamped, w.double(), Hkv)
+    k_o2.backward(gk.double())
+    torch.autograd.backward((k, v), (gk.to(DEV), gk.to(DEV)))
+    ref = ck_o.grad
+    assert (ck_g.grad.double().cpu() - ref).abs().max().item() <= 4e-3 * ref.abs().max().item()
+
+
+def test_store_with_spare_capacity_is_read_in_place_and_the_cache_uses_the_kernel():
+    import gca_hip
+    from gca_hip.chunk_cache import ChunkKVManager
+    N, C, S, Dm, K = 2, 6, 64, 128, 3
+    ck, cv, idx, w = _case(N, C, S, Dm, K, torch.bfloat16, 90)
+    store_k = torch.zeros(N, 16, S, Dm, device=DEV, dtype=torch.bfloat16)
+    store_v = torch.zeros_like(store_k)
+    store_k[:, :C], store_v[:, :C] = ck.to(DEV), cv.to(DEV)
+    k_o, v_o, _ = orc.gather_chunks(ck, cv, idx, w, 2)
+    k, v, _ = gca_hip.gather_chunks(store_k[:, :C], store_v[:, :C], idx.to(DEV), w.to(DEV), 2)
+    assert torch.equal(k.cpu(), k_o) and torch.equal(v.cpu(), v_o)
+    # retrieve_chunks of the cache object: rows stay whole (DRT.py:193-200)
+    cache = ChunkKVManager(capacity=16)
+    cache.append(ck.to(DEV), cv.to(DEV), gen((N, C, 32), 91, 1.0, torch.bfloat16).to(DEV))
+    sel = torch.tensor([[0, 5, 2, 2], [4, 1, 0, 3]])
+    rk, rv = cache.retrieve_chunks(sel.to(DEV))
+    b = torch.arange(N).unsqueeze(1)
+    assert torch.equal(rk.cpu(), ck[b, sel]) and torch.equal(rv.cpu(), cv[b, sel])
+
+
+def test_arguments_are_checked():
+    from gca_hip import _lib
+    from gca_hip.gca import _ptr, _stream
+    L = _lib.lib()
+    t = torch.zeros(1, 2, 4, 64, device=DEV, dtype=torch.bfloat16)
+    idx = torch.zeros(1, 1, device=DEV, dtype=torch.int64)
+    out = torch.zeros(1, 1, 1, 4, 64, device=DEV, dtype=torch.bfloat16)
+    good = _lib.ChunkGatherDesc(dtype=1, Hkv=1, N=1, C=2, Z=1, K=1, S=4, D=64)
+    assert L.gca_gather_chunks(ctypes.byref(good), _ptr(t), _ptr(t), _ptr(idx), _ptr(out), _ptr(out), _stream(t.device)) == 0
+    assert L.gca_gather_chunks(ctypes.byref(good), None, _ptr(t), _ptr(idx), _ptr(out), _ptr(out), None) == 1
+    odd = _lib.ChunkGatherDesc(dtype=1, Hkv=1, N=1, C=2, Z=1, K=1, S=4, D=12)            # 24-byte rows
+    assert L.gca_gather_chunks(ctypes.byref(odd), _ptr(t), _ptr(t), _ptr(idx), _ptr(out), _ptr(out), None) == _lib.GCA_ERR_SHAPE
+    ragged = _lib.ChunkGatherDesc(dtype=1, Hkv=1, N=2, C=2, Z=3, K=1, S=4, D=64)         # Z % N != 0
+    assert L.gca_scatter_workspace_bytes(ctypes.byref(ragged)) == 0
+    need = L.gca_scatter_workspace_bytes(ctypes.byref(good))
+    assert need > 0
+    assert L.gca_scatter_chunks(ctypes.byref(good), _ptr(out), _ptr(out), _ptr(idx), _ptr(t), _ptr(t), None, 0, None) == 5
+    torch.cuda.synchronize()
