@@ -118,12 +118,26 @@ chunk_gather_kernel(GatherArgs a, const u32x4* __restrict__ k_cache, const u32x4
     const int row = a.Hkv * a.ppr;                       // pieces per cache row
     const int64_t src0 = (n * a.C + c) * a.S * row;
     const int total = a.S * row;
-    for (int i = blockIdx.y * 256 + threadIdx.x; i < total; i += gridDim.y * 256) {
-        const int s = i / row, r = i - s * row;
-        const int hk = r / a.ppr, pp = r - hk * a.ppr;
-        const int64_t dst = (((z * a.Hkv + hk) * a.K + j) * a.S + s) * a.ppr + pp;
-        k_out[dst] = k_cache[src0 + i];
-        v_out[dst] = v_cache[src0 + i];
+    // four pieces of each tensor in flight per thread
+    const int step = gridDim.y * 256;
+    for (int i0 = blockIdx.y * 256 + threadIdx.x; i0 < total; i0 += 4 * step) {
+        u32x4 kq[4], vq[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int i = i0 + u * step;
+            if (i < total) { kq[u] = k_cache[src0 + i]; vq[u] = v_cache[src0 + i]; }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int i = i0 + u * step;
+            if (i < total) {
+                const int s = i / row, r = i - s * row;
+                const int hk = r / a.ppr, pp = r - hk * a.ppr;
+                const int64_t dst = (((z * a.Hkv + hk) * a.K + j) * a.S + s) * a.ppr + pp;
+                k_out[dst] = kq[u];
+                v_out[dst] = vq[u];
+            }
+        }
     }
 }
 
@@ -165,6 +179,7 @@ chunk_scatter_kernel(GatherArgs a, const E* __restrict__ dk_g, const E* __restri
                 s_tile[tid] = ((z * a.Hkv + hk) * a.K + j) * (int64_t)tile;
             }
             __syncthreads();
+#pragma unroll 4
             for (int ri = 0; ri < nb; ++ri) {
                 const int64_t base = s_tile[ri];
 #pragma unroll
