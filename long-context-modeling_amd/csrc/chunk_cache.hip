@@ -99,8 +99,6 @@ int launch_chunk_append(const chunk_cache_desc& d, const void* sk, const void* s
 // d[z, hk, j, s, :], walked in the reference lists' fixed order, accumulated in float, every cache element
 // written exactly once (zeros where nobody retrieved the chunk): no atomics, no zero-fill, same bits every run.
 
-namespace {
-
 struct GatherArgs {
     int64_t N, C, Z, zpn;
     int K, S, Hkv, D;
@@ -221,7 +219,7 @@ chunk_scatter_kernel(GatherArgs a, const E* __restrict__ dk_g, const E* __restri
     }
 }
 
-GatherArgs gather_args(const chunk_gather_desc& d) {
+static GatherArgs gather_args(const chunk_gather_desc& d) {
     GatherArgs a;
     a.N = d.N; a.C = d.C; a.Z = d.Z; a.zpn = d.Z / d.N;
     a.K = d.K; a.S = d.S; a.Hkv = d.Hkv; a.D = d.D;
@@ -230,7 +228,7 @@ GatherArgs gather_args(const chunk_gather_desc& d) {
 }
 
 // the list builders only look at the retrieval's shape
-Params list_params(const chunk_gather_desc& d) {
+static Params list_params(const chunk_gather_desc& d) {
     Params p = {};
     p.Z = d.Z; p.N = d.N; p.C = d.C; p.zpn = d.Z / d.N; p.K = d.K;
     p.Hkv = d.Hkv; p.K_CTX = d.S; p.D = d.D; p.indexed = 1;
@@ -238,8 +236,6 @@ Params list_params(const chunk_gather_desc& d) {
 }
 
 constexpr int SCATTER_SEG_MAX = 1 << 30;     // the scatter walks every chunk's list whole
-
-}  // namespace
 
 int launch_chunk_gather(const chunk_gather_desc& d, const void* k_cache, const void* v_cache, const int64_t* indices,
                         void* k_out, void* v_out, hipStream_t s) {
