@@ -161,7 +161,7 @@ chunk_scatter_kernel(GatherArgs a, const E* __restrict__ dk_g, const E* __restri
     const int tile = a.S * a.D;
     const int pieces = tile / V;
     // a thread owns pieces tid, tid + 256, ...; NP of them are carried through a batch of references at a time
-    constexpr int NP = 4;
+    constexpr int NP = 2;
     for (int pbase = 0; pbase < pieces; pbase += 256 * NP) {      // uniform bounds: the loop body has barriers
         const int p0 = pbase + tid;
         float acc_k[NP][V], acc_v[NP][V];
@@ -177,7 +177,7 @@ chunk_scatter_kernel(GatherArgs a, const E* __restrict__ dk_g, const E* __restri
                 s_tile[tid] = ((z * a.Hkv + hk) * a.K + j) * (int64_t)tile;
             }
             __syncthreads();
-#pragma unroll 4
+#pragma unroll 8
             for (int ri = 0; ri < nb; ++ri) {
                 const int64_t base = s_tile[ri];
 #pragma unroll
