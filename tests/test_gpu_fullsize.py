@@ -215,6 +215,12 @@ def test_cfg2_indexed_equals_gathered():
     flat = (idx + (torch.arange(Z, device=DEV) // (C - 1) * C)[:, None]).view(-1)
     ref.index_add_(0, flat, dkg.float().permute(0, 2, 3, 1, 4).reshape(Z * K, S, H, d))
     assert _rel(dkc.view(N * C, S, H, d), ref) <= 2e-2
+    # and the gather's own backward (the scatter kernel) gives that sum to bf16 rounding
+    ck_g, cv_g = ck.clone().requires_grad_(True), cv.clone().requires_grad_(True)
+    kg2, vg2, _ = gca_hip.gather_chunks(ck_g, cv_g, indices, weights, H)
+    assert torch.equal(kg2, kg) and torch.equal(vg2, vg)
+    dck, dcv = torch.autograd.grad((kg2, vg2), (ck_g, cv_g), (dkg, dvg))
+    assert _rel(dck.view(N * C, S, H, d), ref) <= 4e-3
 
 
 def test_cfg4_geometry_mfma_vs_generic():
